@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (``architectures[0]`` of config.json) to its
+"""One registry from an architecture's name (``architectures[0]`` or ``architecture`` of config.json) to its
 typed configuration and the function that turns it into a ``ModelSpec``.
 
 The reference keeps a list of (name, constructor) pairs and answers an unknown name with
@@ -50,7 +50,10 @@ def read_config(source):
         path = os.path.join(source, "config.json") if os.path.isdir(source) else source
         with open(path, "r", encoding="utf-8") as fh:
             raw = json.load(fh)
+    # ``architectures`` (a list, the first counts), also under ``text_config``, or ``architecture`` (one name)
     archs = raw.get("architectures") or raw.get("text_config", {}).get("architectures") or []
+    if not archs and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]
     if not archs:
         raise UnknownArchitecture(f"config names no architecture; registered: {sorted(_ARCHITECTURES)}")
     arch = architecture(archs[0])

@@ -127,6 +127,20 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// The gate's activation in a gated product act(gate) * up: SP_ACT_SILU g * sigmoid(g), or
+// SP_ACT_GELU_TANH 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).  `fast`: the short exponential
+// (the bfloat16 products); the 32-bit path takes the accurate routines.
+enum { SP_ACT_NONE = 0, SP_ACT_SILU = 1, SP_ACT_GELU_TANH = 2 };
+__device__ __forceinline__ float sp_gate_act(float g, int act, bool fast) {
+    if (act == SP_ACT_GELU_TANH) {
+        const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+        // tanh(z) = 1 - 2 / (exp(2z) + 1): no cancellation where it matters, exact limits at both ends
+        const float t = fast ? 1.0f - 2.0f / (__expf(2.0f * z) + 1.0f) : tanhf(z);
+        return 0.5f * g * (1.0f + t);
+    }
+    return g / (1.0f + (fast ? __expf(-g) : expf(-g)));
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<bf16>(bf16 v) { return (float)v; }

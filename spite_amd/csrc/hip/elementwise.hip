@@ -77,6 +77,10 @@ __device__ __forceinline__ float wave_dot_row(const float* __restrict__ w, const
 // With `proj` ([P, d] fp32) the normed fp32 row also goes to LDS and the waves form its P
 // products proj . y into proj_out[i][0..P): the router's logits, without the row going to
 // memory in 32-bit and back.
+// With `dn` (fp32 rows like d1) a further increment is normed on its way in:
+// v += mult * dn[r] * 1/sqrt(mean(dn[r]^2) + eps_n) * wn  (a sublayer's result that passes a norm
+// of its own and a constant before it joins the residual stream).  With `plain_out`, out[i] is v
+// itself in the output's dtype (no norm, `w` unused): the stream as a later product's operand.
 #define NORM_NT 512
 #define NORM_MAX_V 8     // widths up to 4*NT*MAX_V = 16384 stay in registers
 template <typename TO, bool VEC>
@@ -85,7 +89,9 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                         const float* __restrict__ d2, const float* __restrict__ w,
                         TO* __restrict__ out, float* __restrict__ out32,
                         const int* __restrict__ rows, int d, float eps, int write_h,
-                        const float* __restrict__ proj, float* __restrict__ proj_out, int P) {
+                        const float* __restrict__ proj, float* __restrict__ proj_out, int P,
+                        const float* __restrict__ dn, const float* __restrict__ wn, float mult, float eps_n,
+                        int plain_out) {
     __shared__ float red[NORM_NT / 64];
     extern __shared__ __attribute__((aligned(16))) float ys[];            // [d] if proj
     const int i = blockIdx.x;
@@ -93,11 +99,26 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
     float* hr = h + r * d;
     const float* a = d1 ? d1 + r * d : nullptr;
     const float* b = d2 ? d2 + r * d : nullptr;
+    const float* nr = dn ? dn + r * d : nullptr;
     float ss = 0.f;
     if (VEC) {
         // d is a multiple of 4 and at most 4*NT*MAX_V
         f32x4 v[NORM_MAX_V];
         const int nv = d >> 2;
+        float sn = 0.f;
+        if (nr) {
+            float sq = 0.f;
+#pragma unroll
+            for (int u = 0; u < NORM_MAX_V; ++u) {
+                const int c = threadIdx.x + u * NORM_NT;
+                if (c < nv) {
+                    const f32x4 x = ((const f32x4*)nr)[c];
+                    v[u] = x;
+                    sq += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+                }
+            }
+            sn = mult / sqrtf(block_sum<NORM_NT>(sq, red) / (float)d + eps_n);
+        }
 #pragma unroll
         for (int u = 0; u < NORM_MAX_V; ++u) {
             const int c = threadIdx.x + u * NORM_NT;
@@ -105,21 +126,29 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                 f32x4 x = ((const f32x4*)hr)[c];
                 if (a) x += ((const f32x4*)a)[c];
                 if (b) x += ((const f32x4*)b)[c];
+                if (nr) {
+                    const f32x4 ww = ((const f32x4*)wn)[c];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[e] += v[u][e] * sn * ww[e];
+                }
                 if (write_h) ((f32x4*)hr)[c] = x;
                 v[u] = x;
                 ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
             }
         }
+        if (!out && !out32 && !proj) return;               // the additions were all that was asked for
         const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
         const float scale = 1.0f / sqrtf(ms + eps);
 #pragma unroll
         for (int u = 0; u < NORM_MAX_V; ++u) {
             const int c = threadIdx.x + u * NORM_NT;
             if (c < nv) {
-                const f32x4 ww = ((const f32x4*)w)[c];
-                f32x4 y;
+                f32x4 y = v[u];
+                if (!plain_out) {
+                    const f32x4 ww = ((const f32x4*)w)[c];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) y[e] = v[u][e] * scale * ww[e];
+                    for (int e = 0; e < 4; ++e) y[e] = v[u][e] * scale * ww[e];
+                }
                 if (out32) ((f32x4*)(out32 + (size_t)i * d))[c] = y;
                 if (proj) ((f32x4*)ys)[c] = y;
                 if (out) {
@@ -135,19 +164,27 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
             }
         }
     } else {
+        float sn = 0.f;
+        if (nr) {
+            float sq = 0.f;
+            for (int c = threadIdx.x; c < d; c += NORM_NT) sq += nr[c] * nr[c];
+            sn = mult / sqrtf(block_sum<NORM_NT>(sq, red) / (float)d + eps_n);
+        }
         for (int c = threadIdx.x; c < d; c += NORM_NT) {
             float x = hr[c];
             if (a) x += a[c];
             if (b) x += b[c];
+            if (nr) x += nr[c] * sn * wn[c];
             if (write_h) hr[c] = x;
             ss += x * x;
         }
+        if (!out && !out32 && !proj) return;
         const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
         const float scale = 1.0f / sqrtf(ms + eps);
         for (int c = threadIdx.x; c < d; c += NORM_NT) {
             float x = hr[c];
-            if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; }
-            const float y = x * scale * w[c];
+            if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; if (nr) x += nr[c] * sn * wn[c]; }
+            const float y = plain_out ? x : x * scale * w[c];
             if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
             if (out32) out32[(size_t)i * d + c] = y;
             if (proj) ys[c] = y;
@@ -167,16 +204,19 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
 extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, const float* w, void* out,
                                  int out_dtype, float* out32, const int* rows, int n_rows, int d,
                                  float eps, int write_h, const float* proj, float* proj_out, int P,
+                                 const float* dn, const float* wn, float mult, float eps_n, int plain_out,
                                  hipStream_t st) {
     SP_REQUIRE(n_rows >= 0 && d > 0 && eps > 0.f, "add_rmsnorm: bad sizes rows=%d d=%d eps=%g", n_rows, d, eps);
+    SP_REQUIRE(!dn || (wn && eps_n > 0.f), "add_rmsnorm: a normed increment needs its weight and eps");
+    SP_REQUIRE(w || plain_out || (!out && !out32 && !proj), "add_rmsnorm: a normed output needs the norm's weight");
     SP_REQUIRE(!proj || (proj_out && P > 0), "add_rmsnorm: a projection needs its output and size");
     const size_t sh = proj ? (size_t)d * sizeof(float) : 0;
     SP_REQUIRE(sh <= 48 * 1024, "add_rmsnorm: rows of %d do not fit the projection's LDS", d);
     if (n_rows == 0) return 0;
     auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
-    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32) && al(out);
-#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); \
-        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P); } while (0)
+    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32) && al(out) && al(dn) && al(wn);
+#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out); \
+        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out); } while (0)
     if (out_dtype == SP_F32) SP_NORM(float);
     else if (out_dtype == SP_BF16) SP_NORM(bf16);
     else return sp_fail("add_rmsnorm: unknown dtype %d", out_dtype);
@@ -576,7 +616,7 @@ __device__ __forceinline__ int top1_of(const float* __restrict__ l, int E, float
 __global__ void moe_plan_kernel(int* __restrict__ expert, float* __restrict__ weight,
                                 const float* __restrict__ logits,
                                 int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
-                                int* __restrict__ offsets, int T, int E, int shared) {
+                                int* __restrict__ offsets, int T, int E, int shared, int fan) {
     extern __shared__ unsigned short e_of[];
     for (int i = threadIdx.x; i < T; i += blockDim.x)
         e_of[i] = (unsigned short)(logits ? top1_of(logits + (size_t)i * E, E, nullptr) : expert[i]);
@@ -598,7 +638,7 @@ __global__ void moe_plan_kernel(int* __restrict__ expert, float* __restrict__ we
             const int ej = e_of[j];
             rank += (ej < me) || (ej == me && j < t);
         }
-        src[rank] = t; scale[rank] = wt; dst[rank] = t;
+        src[rank] = t / fan; scale[rank] = wt; dst[rank] = t;
         if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
     }
     if (blockIdx.x == 0) {
@@ -621,7 +661,7 @@ __global__ __launch_bounds__(256)
 void moe_plan_hist_kernel(int* __restrict__ expert, float* __restrict__ weight,
                           const float* __restrict__ logits,
                           int* __restrict__ src, float* __restrict__ scale, int* __restrict__ dst,
-                          int* __restrict__ offsets, int T, int E, int shared) {
+                          int* __restrict__ offsets, int T, int E, int shared, int fan) {
     extern __shared__ int sh[];              // total[E], before[E], first[E+1], mine[256]
     int* total = sh; int* before = sh + E; int* first = sh + 2 * E; int* mine = sh + 3 * E + 1;
     const int c0 = blockIdx.x * 256, t = c0 + threadIdx.x;
@@ -656,7 +696,7 @@ void moe_plan_hist_kernel(int* __restrict__ expert, float* __restrict__ weight,
     if (t < T && (unsigned)me < (unsigned)E) {
         int rank = first[me] + before[me];
         for (int j = 0; j < (int)threadIdx.x; ++j) rank += mine[j] == me;
-        src[rank] = t; scale[rank] = wt; dst[rank] = t;
+        src[rank] = t / fan; scale[rank] = wt; dst[rank] = t;
         if (shared) { src[T + t] = t; scale[T + t] = 1.0f; dst[T + t] = T + t; }
     }
     if (blockIdx.x == 0) {
@@ -666,17 +706,21 @@ void moe_plan_hist_kernel(int* __restrict__ expert, float* __restrict__ weight,
 }
 
 // `logits` null: expert[] and weight[] are inputs; else they are outputs.
+// `fan` > 1: the T entries are the choices of T / fan tokens, `fan` in a row for each (a router
+// that takes several experts a token); src[] then names the token, entry / fan, that a slot reads
+// its input row from, while dst[] stays the entry: every choice has an output row of its own.
 extern "C" int spite_moe_plan(int* expert, float* weight, const float* logits, int* src, float* scale, int* dst,
-                              int* offsets, int T, int E, int shared, hipStream_t st) {
+                              int* offsets, int T, int E, int shared, int fan, hipStream_t st) {
     SP_REQUIRE(T >= 0 && E > 0 && E < 65535, "moe_plan: bad sizes T=%d E=%d", T, E);
-    SP_REQUIRE(T <= 32768, "moe_plan: %d tokens in one step, at most 32768", T);
+    SP_REQUIRE(fan >= 1 && (fan == 1 || (!shared && !logits)), "moe_plan: a fan of %d goes with given experts and no shared group", fan);
+    SP_REQUIRE(T <= ((T > 256 && E <= PLAN_MAX_E) ? (1 << 22) : 32768), "moe_plan: %d entries in one step are too many", T);
     const int grid = T > 0 ? (T + 255) / 256 : 1;
     if (T > 256 && E <= PLAN_MAX_E)
         moe_plan_hist_kernel<<<grid, 256, (size_t)(3 * E + 1 + 256) * sizeof(int), st>>>(
-            expert, weight, logits, src, scale, dst, offsets, T, E, shared);
+            expert, weight, logits, src, scale, dst, offsets, T, E, shared, fan);
     else
         moe_plan_kernel<<<grid, 256, (size_t)(T > 0 ? T : 1) * sizeof(unsigned short), st>>>(
-            expert, weight, logits, src, scale, dst, offsets, T, E, shared);
+            expert, weight, logits, src, scale, dst, offsets, T, E, shared, fan);
     SP_LAUNCH_CHECK("moe_plan");
     return 0;
 }

@@ -7,7 +7,7 @@
 // [offsets[g], offsets[g+1]) and multiplies them with W + g*w_group_stride.  A slot reads
 // row a_rows[s] of A (times a_scale[s], in fp32, before the product) and writes row
 // y_rows[s] of Y.  With `glu` the group's W holds 2N rows, gate rows first, and the kernel
-// writes silu(gate) * up.
+// writes act(gate) * up (`glu`: 1 silu, 2 the tanh form of gelu).
 #include "common.h"
 
 #define GBM 64
@@ -20,7 +20,7 @@ void gemm_generic_kernel(const T* __restrict__ A, int lda, const T* __restrict__
                          TY* __restrict__ Y, int ldy, int M, int N, int K,
                          const int* __restrict__ offsets, int n_groups,
                          const int* __restrict__ a_rows, const float* __restrict__ a_scale,
-                         const int* __restrict__ y_rows) {
+                         const int* __restrict__ y_rows, int act) {
     __shared__ float As[GBK][GBM + 1];
     __shared__ float Ws[GLU ? 2 : 1][GBK][GBN + 1];
     // ---- which group and which of its row tiles
@@ -88,7 +88,7 @@ void gemm_generic_kernel(const T* __restrict__ A, int lda, const T* __restrict__
             const int n = n0 + tn + j;
             if (n >= N) continue;
             float v = acc_g[i][j];
-            if (GLU) v = v / (1.0f + expf(-v)) * acc_u[i][j];
+            if (GLU) v = sp_gate_act(v, act, false) * acc_u[i][j];
             Y[yr * ldy + n] = from_f32<TY>(v);
         }
     }
@@ -107,7 +107,7 @@ extern "C" int spite_gemm_generic(const void* A, int lda, const void* W, long w_
     SP_REQUIRE(m_tiles <= 65535, "gemm: too many row tiles (%d)", m_tiles);
     dim3 grid((N + GBN - 1) / GBN, m_tiles);
 #define SP_GEMM_LAUNCH(T, TY, GLU) gemm_generic_kernel<T, TY, GLU><<<grid, 256, 0, st>>>( \
-        (const T*)A, lda, (const T*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows)
+        (const T*)A, lda, (const T*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, glu)
     if (dtype == SP_F32 && y_dtype == SP_F32) { if (glu) SP_GEMM_LAUNCH(float, float, 1); else SP_GEMM_LAUNCH(float, float, 0); }
     else if (dtype == SP_BF16 && y_dtype == SP_BF16) { if (glu) SP_GEMM_LAUNCH(bf16, bf16, 1); else SP_GEMM_LAUNCH(bf16, bf16, 0); }
     else if (dtype == SP_BF16 && y_dtype == SP_F32) { if (glu) SP_GEMM_LAUNCH(bf16, float, 1); else SP_GEMM_LAUNCH(bf16, float, 0); }

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                       TY* __restrict__ Y, int ldy, int M, int N, int K,
                       const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
-                      const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles) {
+                      const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles, int act) {
     static_assert(WN * WM == 8, "eight waves");
     constexpr int BM = 128 * WM, BN = 64 * WN;
     constexpr int NCOLS = GLU ? BN / 2 : BN;        // output columns per workgroup
@@ -164,7 +164,7 @@ void gemm_mfma_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restric
                 for (int i = 0; i < 4; ++i) {
                     if (n + i < N) {
                         const float gv = acc[a][b][i] * sc, uv = acc[a + TG][b][i] * sc;
-                        yrow[n + i] = from_f32<TY>(gv / (1.0f + __expf(-gv)) * uv);
+                        yrow[n + i] = from_f32<TY>(sp_gate_act(gv, act, true) * uv);
                     }
                 }
             }
@@ -192,9 +192,9 @@ static int launch_mfma(const void* X, int ldx, const void* W, long w_group_strid
     SP_REQUIRE((long)m_tiles * n_tiles < (1L << 30), "gemm_mfma: too many tiles");
     dim3 grid((m_tiles * n_tiles + 7) / 8 * 8);
 #define SP_MM(GLUV, TY) do { if (K % MBK == 0) gemm_mfma_kernel<WN, WM, GLUV, true, TY><<<grid, 512, 0, st>>>((const bf16*)X, ldx, \
-        (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, m_tiles, n_tiles); \
+        (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, m_tiles, n_tiles, glu); \
     else gemm_mfma_kernel<WN, WM, GLUV, false, TY><<<grid, 512, 0, st>>>((const bf16*)X, ldx, (const bf16*)W, \
-        w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, m_tiles, n_tiles); } while (0)
+        w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, m_tiles, n_tiles, glu); } while (0)
     if (glu) { if (y_dtype == SP_BF16) SP_MM(true, bf16); else SP_MM(true, float); }
     else { if (y_dtype == SP_BF16) SP_MM(false, bf16); else SP_MM(false, float); }
 #undef SP_MM

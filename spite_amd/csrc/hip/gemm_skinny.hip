@@ -32,7 +32,7 @@ __global__ __launch_bounds__(NW * 64)
 void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restrict__ W, long w_group_stride,
                         TY* __restrict__ Y, int ldy, int M, int N, int K,
                         const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
-                        const float* __restrict__ a_scale, const int* __restrict__ y_rows) {
+                        const float* __restrict__ a_scale, const int* __restrict__ y_rows, int act) {
     constexpr int RA = GLU ? 2 * R : R;        // A tiles per wave
     constexpr int KB = 32 * S;                 // k elements per block
     constexpr int J = RA * G * 4;              // partial sums per lane
@@ -156,7 +156,7 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
             if (GLU) u += red[(w * J + j + JO) * 64 + l];
         }
         if (a_scale) { const float sc = a_scale[s]; v *= sc; u *= sc; }
-        if (GLU) v = v / (1.0f + __expf(-v)) * u;
+        if (GLU) v = sp_gate_act(v, act, true) * u;
         const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
         Y[yr * ldy + n] = from_f32<TY>(v);
     }
@@ -181,7 +181,7 @@ static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* 
         if (sh > 48 * 1024) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
             if (e != hipSuccess) return sp_fail("gemm_skinny: cannot get %zu bytes of LDS: %s", sh, hipGetErrorString(e)); } \
         kern<<<grid, NW * 64, sh, st>>>((const bf16*)X, ldx, (const bf16*)W, wgs, (TY*)Y, ldy, M, N, K, offsets, \
-                                        n_groups, a_rows, a_scale, y_rows); } while (0)
+                                        n_groups, a_rows, a_scale, y_rows, glu); } while (0)
     if (glu) { if (y_dtype == SP_BF16) SP_SK(true, bf16); else SP_SK(true, float); }
     else { if (y_dtype == SP_BF16) SP_SK(false, bf16); else SP_SK(false, float); }
 #undef SP_SK

@@ -39,7 +39,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
                        TY* __restrict__ Y, int ldy, int M, int N, int K,
                        const int* __restrict__ offsets, int n_groups, const int* __restrict__ a_rows,
                        const float* __restrict__ a_scale, const int* __restrict__ y_rows, int m_tiles, int n_tiles,
-                       int k_splits, size_t split_stride) {
+                       int k_splits, size_t split_stride, int act) {
     static_assert(WN * WM == 8, "eight waves");
     constexpr int WS = 16 * NB;                     // slots of a wave: NB slot tiles
     constexpr int BM = WS * WM, BN = 64 * WN;
@@ -267,7 +267,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float gv = acc[a][b][i] * sc, uv = acc[a + TG][b][i] * sc;
-                    v[i] = gv / (1.0f + __expf(-gv)) * uv;
+                    v[i] = sp_gate_act(gv, act, true) * uv;
                 }
                 put4(yrow, ncol[a] + q * 4, v);
             }
@@ -282,6 +282,10 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
         }
     }
 }
+
+// The gate's activation of the gated product that the calling thread is launching (set by the
+// entry point; the launchers below hand it to the kernel).
+static thread_local int g_gate_act = SP_ACT_SILU;
 
 template <int WN, int WM, int NB, bool GLU, typename TY, bool NTW = false>
 static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_group_stride, void* Y, int ldy, int M, int N,
@@ -308,11 +312,11 @@ static int launch_tiled_kernel(const void* X, int ldx, const void* W, long w_gro
     if (offsets)
         gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, true><<<grid, 512, sh, st>>>(
             (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
-            y_rows, m_tiles, n_tiles, k_splits, split_stride);
+            y_rows, m_tiles, n_tiles, k_splits, split_stride, g_gate_act);
     else
         gemm_tiled_kernel<WN, WM, NB, GLU, TY, NTW, false><<<grid, 512, sh, st>>>(
             (const bf16*)X, ldx, (const bf16*)W, w_group_stride, (TY*)Y, ldy, M, N, K, offsets, n_groups, a_rows, a_scale,
-            y_rows, m_tiles, n_tiles, k_splits, split_stride);
+            y_rows, m_tiles, n_tiles, k_splits, split_stride, g_gate_act);
     SP_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
@@ -389,6 +393,7 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
     SP_REQUIRE(shape >= 0 && shape <= 6, "gemm_tiled: tile shape %d", shape);
+    g_gate_act = glu ? glu : SP_ACT_SILU;
     if (M == 0) return 0;
     if (shape == 0) {
         // Tiles come in whole numbers per CU: a plain product whose 128-row tiles leave many of the

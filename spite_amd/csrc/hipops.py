@@ -17,6 +17,8 @@ from . import build
 
 F32, BF16 = 0, 1
 VIS = build.visibility_codes()      # "full", "chunk", "window": name -> code
+# the gate's activation of a gated product act(gate) * up, as the kernels number them (True: silu)
+GATE_ACTS = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 2}
 
 
 class KernelError(RuntimeError):
@@ -34,10 +36,10 @@ def lib():
         P, I, L, F = c_void_p, c_int, c_long, c_float
         sigs = {
             "spite_embed": [P, P, I, P, I, I, I, P],
-            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P],
+            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P, P, F, F, I, P],
             "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, I, P, P, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
-            "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, P],
+            "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, I, P],
             "spite_convert": [P, I, P, I, c_size_t, P],
             "spite_add_into": [P, P, c_size_t, P],
             "spite_randn_fill": [P, I, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, F, F, P],
@@ -55,6 +57,11 @@ def lib():
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
             "spite_mfma_loop": [P, I, I, F, P],
+            "spite_latent_prepare": [P, I, P, I, P, P, I, P, P, P, P, F, I, I, I, I, I, I, I, P, P, P],
+            "spite_attn_latent_generic": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
+            "spite_router_topk": [P, P, P, P, I, I, I, I, P],
+            "spite_moe_combine": [P, P, P, P, I, I, I, P],
+            "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -90,6 +97,14 @@ def _ptr(t, name, dtype=None, optional=False):
     return t.data_ptr()
 
 
+def _ptr_rows(t, name):
+    """A matrix whose rows may lie apart (a column range of a wider one): the products take the
+    row stride beside the pointer."""
+    if t is not None and t.dim() == 2 and t.is_cuda and t.stride(1) == 1 and t.stride(0) >= t.shape[1]:
+        return t.data_ptr()
+    return _ptr(t, name)
+
+
 def _check_pages(k_pages, v_pages, G, page_size, hd, what):
     """Key pages [n, G, page_size, hd]; value pages transposed, [n, G, hd, page_size]."""
     if (tuple(k_pages.shape[1:]) != (G, page_size, hd) or tuple(v_pages.shape[1:]) != (G, hd, page_size)
@@ -123,17 +138,27 @@ def add_rmsnorm_can_project(d: int) -> bool:
 
 
 def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True,
-                proj=None, proj_out=None):
+                proj=None, proj_out=None, normed=None, plain_out=False):
     """v = h[r] + d1[r] + d2[r] (stored back if write_h); out[i] = rmsnorm(v) * w with r =
     rows[i] or i.  h, d1, d2, out32 fp32; w fp32 [d]; out fp32 or bf16.  With ``proj`` ([P, d]
     fp32) also proj_out[i] = proj . (the normed row in fp32), [n, P] fp32: the same bits as
-    ``router_top1`` gives for that row."""
+    ``router_top1`` gives for that row.  ``normed`` = (dn, wn, mult, eps_n): a further increment
+    mult * rmsnorm(dn[r]; eps_n) * wn, normed on its way in.  ``plain_out``: out[i] = v itself (no
+    norm; ``w`` may be None).  With no output at all the call only adds."""
     d = h.shape[-1]
+    dn = wn = None
+    mult = eps_n = 0.0
+    if normed is not None:
+        dn, wn, mult, eps_n = normed
+        if dn.shape[-1] != d or dn.shape[0] < h.shape[0] or wn.numel() != d:
+            raise KernelError(f"add_rmsnorm: normed increment {tuple(dn.shape)} with weight of {wn.numel()} for h {tuple(h.shape)}")
+    if w is None and not plain_out and (out is not None or out32 is not None or proj is not None):
+        raise KernelError("add_rmsnorm: a normed output needs the norm's weight")
     n = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
     for name, t in (("d1", d1), ("d2", d2)):
         if t is not None and (t.shape[-1] != d or t.shape[0] < h.shape[0]):
             raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} does not match h {tuple(h.shape)}")
-    if w.numel() != d:
+    if w is not None and w.numel() != d:
         raise KernelError(f"add_rmsnorm: weight of {w.numel()} for rows of {d}")
     for name, t in (("out", out), ("out32", out32)):
         if t is not None and (t.shape[-1] != d or t.shape[0] < n):
@@ -148,10 +173,12 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
             raise KernelError("add_rmsnorm: projection [P, d] with an output [rows, P]")
     _check(lib().spite_add_rmsnorm(
         _ptr(h, "h", torch.float32), _ptr(d1, "d1", torch.float32, True), _ptr(d2, "d2", torch.float32, True),
-        _ptr(w, "w", torch.float32), _ptr(out, "out", None, True),
+        _ptr(w, "w", torch.float32, True), _ptr(out, "out", None, True),
         dtype_code(out.dtype) if out is not None else F32, _ptr(out32, "out32", torch.float32, True),
         _ptr(rows, "rows", torch.int32, True), n, d, float(eps), int(write_h),
-        _ptr(proj, "proj", torch.float32, True), _ptr(proj_out, "proj_out", torch.float32, True), P, _stream()),
+        _ptr(proj, "proj", torch.float32, True), _ptr(proj_out, "proj_out", torch.float32, True), P,
+        _ptr(dn, "normed increment", torch.float32, True), _ptr(wn, "normed increment's weight", torch.float32, True),
+        float(mult), float(eps_n), int(bool(plain_out)), _stream()),
         "add_rmsnorm")
 
 
@@ -207,9 +234,11 @@ def router_top1(x32, w_router, expert, weight, logits_out=None):
            "router_top1")
 
 
-def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared, logits=None):
+def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared, logits=None, fan=1):
     """Row list of the grouped products from the router's choice (see the kernel).  With
-    ``logits`` ([T, E] fp32) the choice is made here and written to ``expert`` and ``weight``."""
+    ``logits`` ([T, E] fp32) the choice is made here and written to ``expert`` and ``weight``.
+    ``fan`` > 1: the T entries are ``fan`` choices in a row for each of T / fan tokens; ``src`` names
+    the token (entry // fan), ``dst`` the entry."""
     n = 2 * T if shared else T
     if src.numel() < n or scale.numel() < n or dst.numel() < n or offsets.numel() < E + 1 + int(bool(shared)):
         raise KernelError("moe_plan: output arrays too small")
@@ -220,7 +249,7 @@ def moe_plan(expert, weight, src, scale, dst, offsets, T, E, shared, logits=None
     _check(lib().spite_moe_plan(_ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
                                 _ptr(logits, "logits", torch.float32, True), _ptr(src, "src", torch.int32), _ptr(scale, "scale", torch.float32),
                                 _ptr(dst, "dst", torch.int32), _ptr(offsets, "offsets", torch.int32),
-                                T, E, int(bool(shared)), _stream()), "moe_plan")
+                                T, E, int(bool(shared)), int(fan), _stream()), "moe_plan")
 
 
 def convert(src, dst):
@@ -270,8 +299,8 @@ def gemm_generic(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_s
     if w.dtype != a.dtype:
         raise KernelError(f"gemm: activations {a.dtype} against weights {w.dtype}")
     _check(lib().spite_gemm_generic(
-        _ptr(a, "a"), a.stride(0) if a.dim() == 2 else K, _ptr(w, "w"), rows_w * K, dtype_code(a.dtype),
-        _ptr(y, "y"), dtype_code(y.dtype), y.stride(0), M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups,
+        _ptr_rows(a, "a"), a.stride(0) if a.dim() == 2 else K, _ptr(w, "w"), rows_w * K, dtype_code(a.dtype),
+        _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0), M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups,
         _ptr(a_rows, "a_rows", torch.int32, True), _ptr(a_scale, "a_scale", torch.float32, True),
         _ptr(y_rows, "y_rows", torch.int32, True), int(glu), _stream()), "gemm")
 
@@ -355,7 +384,7 @@ def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sc
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_skinny: bfloat16 operands only, got {a.dtype} and {w.dtype}")
     _check(lib().spite_gemm_skinny(
-        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        _ptr_rows(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
         int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), int(live_groups), _stream()),
@@ -419,7 +448,7 @@ def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scal
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_mfma: bfloat16 operands only, got {a.dtype} and {w.dtype}")
     _check(lib().spite_gemm_mfma(
-        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        _ptr_rows(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
         int(shape), _stream()), "gemm_mfma")
@@ -482,7 +511,7 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
                                             _stream()), "gemm_tiled")
         return
     _check(lib().spite_gemm_tiled(
-        _ptr(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr(y, "y"), dtype_code(y.dtype), y.stride(0),
+        _ptr_rows(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
         _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
         int(shape), _stream()), "gemm_tiled")
@@ -572,3 +601,92 @@ def mfma_loop(out, steps, gain):
     rate with nothing else moving.  Returns the flops done."""
     _check(lib().spite_mfma_loop(_ptr(out, "out", torch.float32), out.numel(), int(steps), float(gain), _stream()), "mfma_loop")
     return out.numel() * 8 * int(steps) * 32 * 16384
+
+
+# -------------------------------------------------------------------------------------------- latent attention
+def latent_prepare(qd, dkv, qa, kv_pages, positions, slot_map, inv_freq, w_norm, eps, H, n, r, R, rot_dims, own,
+                   rows_th, offsets_h):
+    """Between the projections and the per-head products of latent attention (see latent.hip):
+    qd [T, H*(n+r)]; dkv [T, R+r] (with ``own``); qa [T*H, R+r] receives the rotated query parts; with ``own`` the
+    cache row of every token (kv_pages [pages, 1, page_size, R+r]) receives the normed latent and the
+    rotated shared key part; rows_th int32 [H*T] and offsets_h int32 [H+1] receive the row list of
+    the per-head products."""
+    T = qd.shape[0]
+    Dk = R + r
+    if qd.dim() != 2 or qd.stride(1) != 1 or qd.shape[1] < H * (n + r):
+        raise KernelError(f"latent_prepare: qd {tuple(qd.shape)} for H={H} n={n} r={r} R={R} own={own}")
+    if own and (dkv is None or dkv.dim() != 2 or dkv.stride(1) != 1 or dkv.shape[1] < R + r or dkv.shape[0] < T or dkv.dtype != qd.dtype):
+        raise KernelError(f"latent_prepare: the down-projection's rows do not fit R={R} r={r}")
+    if qa.numel() < T * H * Dk or positions.numel() < T or rows_th.numel() < H * T or offsets_h.numel() < H + 1:
+        raise KernelError("latent_prepare: outputs or positions too small")
+    if inv_freq.numel() < rot_dims // 2:
+        raise KernelError("latent_prepare: frequency table shorter than the turning pairs")
+    dt = qd.dtype
+    if own:
+        if kv_pages.dim() != 4 or kv_pages.shape[1] != 1 or kv_pages.shape[3] != Dk or slot_map.numel() < T or w_norm.numel() != R:
+            raise KernelError(f"latent_prepare: pages {tuple(kv_pages.shape)} for rows of {Dk}, or slots / norm weight too small")
+    _check(lib().spite_latent_prepare(
+        _ptr_rows(qd, "qd"), qd.stride(0), _ptr_rows(dkv, "dkv") if own else None, dkv.stride(0) if own else 0, _ptr(qa, "qa", dt), _ptr(kv_pages, "kv_pages", dt, not own), dtype_code(dt),
+        _ptr(positions, "positions", torch.int32), _ptr(slot_map, "slot_map", torch.int32, not own),
+        _ptr(inv_freq, "inv_freq", torch.float32), _ptr(w_norm, "w_norm", torch.float32, not own), float(eps),
+        T, H, n, r, R, int(rot_dims), int(bool(own)), _ptr(rows_th, "rows_th", torch.int32),
+        _ptr(offsets_h, "offsets_h", torch.int32), _stream()), "latent_prepare")
+
+
+def _latent_checks(q, kv_pages, out, positions, seq_of_token, block_table, T, H, Dk, R, what):
+    if q.numel() < T * H * Dk or out.numel() < T * H * R:
+        raise KernelError(f"{what}: q or out too small")
+    if kv_pages.dim() != 4 or kv_pages.shape[1] != 1 or kv_pages.shape[3] != Dk:
+        raise KernelError(f"{what}: pages {tuple(kv_pages.shape)} for rows of {Dk}")
+    if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
+        raise KernelError(f"{what}: metadata too small")
+
+
+def attn_latent_generic(q, kv_pages, out, positions, seq_of_token, block_table, T, H, Dk, R, vis, span, scale):
+    """Attention of T*H query rows [Dk] over cache rows [Dk] whose first R elements are the value:
+    one shared kv head, any mix of portions and single tokens.  out [T*H, R]."""
+    _latent_checks(q, kv_pages, out, positions, seq_of_token, block_table, T, H, Dk, R, "latent attention")
+    dt = q.dtype
+    _check(lib().spite_attn_latent_generic(
+        _ptr(q, "q"), _ptr(kv_pages, "kv_pages", dt), _ptr(out, "out", dt), dtype_code(dt),
+        _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
+        _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, H, Dk, R, kv_pages.shape[2],
+        VIS[vis], int(span or 0), float(scale), _stream()), "latent attention")
+
+
+# -------------------------------------------------------------------------------------------- several experts a token
+def router_topk(logits, bias, expert, weight, top, renorm=False):
+    """From fp32 router logits [T, E]: scores sigmoid(z); the ``top`` experts with the largest
+    score + bias (bias fp32 [E] or None; lowest index among equals) into expert[T*top], their
+    scores (without the bias; divided by their sum with ``renorm``) into weight[T*top]."""
+    T, E = logits.shape
+    if expert.numel() < T * top or weight.numel() < T * top or (bias is not None and bias.numel() != E):
+        raise KernelError("router_topk: outputs too small or bias of the wrong size")
+    _check(lib().spite_router_topk(_ptr(logits, "logits", torch.float32), _ptr(bias, "bias", torch.float32, True),
+                                   _ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
+                                   T, E, int(top), int(bool(renorm)), _stream()), "router_topk")
+
+
+def moe_combine(y, weight, extra, out, T, top):
+    """out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]); all fp32."""
+    d = out.shape[-1]
+    if y.numel() < T * top * d or weight.numel() < T * top or out.numel() < T * d or (extra is not None and extra.numel() < T * d):
+        raise KernelError("moe_combine: arrays too small")
+    _check(lib().spite_moe_combine(_ptr(y, "y", torch.float32), _ptr(weight, "weight", torch.float32),
+                                   _ptr(extra, "extra", torch.float32, True), _ptr(out, "out", torch.float32),
+                                   T, d, int(top), _stream()), "moe_combine")
+
+
+def gated_rows(a, ids, table, col0, g):
+    """g[t] = gelu_tanh(a[t]) * table[ids[t]][col0 : col0 + n]; a, g [T, n] in the run's dtype."""
+    T, n = a.shape
+    if g.numel() < T * n or ids.numel() < T or table.dim() != 2:
+        raise KernelError("gated_rows: arrays too small")
+    _check(lib().spite_gated_rows(_ptr(a, "a"), dtype_code(a.dtype), _ptr(ids, "ids", torch.int32), _ptr(table, "table"),
+                                  dtype_code(table.dtype), table.shape[1], int(col0), _ptr(g, "g", a.dtype), T, n,
+                                  _stream()), "gated_rows")
+
+
+def attn_latent_mfma_ok(Dk, R, page_size) -> bool:
+    """Whether the MFMA kernel of latent attention takes rows of Dk with a latent of R (bfloat16)."""
+    return False

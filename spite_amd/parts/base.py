@@ -65,8 +65,10 @@ class BlockSpec:
     kind: str                    # arrangement, e.g. "prenorm"
     norm1: PartSpec
     mixer: Any                   # a PartSpec; an arrangement with several mixers takes what it likes here (a dict of them)
-    norm2: PartSpec
-    ffn: PartSpec
+    norm2: Optional[PartSpec]
+    ffn: Optional[PartSpec]      # None: the layer has no feed-forward (arrangements that allow it)
+    extra: Dict[str, Any] = field(default_factory=dict)   # what an arrangement has beyond these four: further
+                                                          # parts by name, constants
 
 
 @dataclass(frozen=True)
@@ -180,6 +182,14 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class SideInput(Part):
+    """Something a layer adds to the stream from the step's tokens beside its mixer and feed-forward."""
+
+    def forward(self, h, pending, ctx):
+        """h fp32 [T, d] with ``pending`` not yet added -> the new pending increments."""
+        raise NotImplementedError
+
+
 class Embedding(Part):
     #: the table [V, d] after loading, for a head that is tied to it (None if there is none)
     table = None
@@ -198,10 +208,30 @@ class Head(Part):
         raise NotImplementedError
 
 
+@dataclass
+class NormedIncrement:
+    """An increment of the residual stream that passes a norm of its own and a constant first:
+    h += mult * rmsnorm(y; eps) * weight.  The norm kernel takes one beside its plain increments."""
+    y: torch.Tensor              # fp32 [T, d]
+    weight: torch.Tensor         # fp32 [d]
+    mult: float
+    eps: float
+
+    def as_arg(self):
+        return (self.y, self.weight, self.mult, self.eps)
+
+
 def two_increments(h, pending):
     """A norm adds up to two increments to the residual stream itself; what ``pending`` holds beyond
     two (a feed-forward with three or more results a token, each written by a grouped product
-    to rows of its own) is added to ``h`` here first, in order.  Returns the two for the norm."""
+    to rows of its own) is added to ``h`` here first, in order.  Returns the two for the norm.
+    A ``NormedIncrement`` left by a block whose successor does not take it itself is added here."""
+    if any(isinstance(p, NormedIncrement) for p in pending):
+        from ..csrc import hipops
+        for p in pending:
+            if isinstance(p, NormedIncrement):
+                hipops.add_rmsnorm(h, None, p.eps, normed=p.as_arg())
+        pending = tuple(p for p in pending if not isinstance(p, NormedIncrement))
     if len(pending) > 2:
         from ..csrc import hipops
         for d in pending[2:]:
@@ -259,7 +289,7 @@ def step_array_builder(name: str) -> Callable:
 
 # ----------------------------------------------------------------------------- registries
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {
-    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
+    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {}, "side": {},
 }
 
 

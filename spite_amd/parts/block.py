@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Block, register, build as build_part, two_increments
+from .base import Block, NormedIncrement, register, build as build_part, two_increments
 
 
 @register("block", "prenorm")
@@ -62,3 +62,91 @@ class PreNormBlock(Block):
             n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
         self.norm2.forward(h, n2, d1=delta, out32=None if n2_32 is n2 else n2_32)
         state["pending"] = tuple(self.ffn.forward(n2, n2_32, ctx))
+
+
+@register("block", "sandwich")
+class SandwichBlock(Block):
+    """Every sublayer has a norm before it and one after it, and its normed result joins the
+    stream times a constant m:  h += m * norm1b(mixer(norm1(h)));  h += m * norm2b(ffn(norm2(h)));
+    then, if the layer has one, a side input from the step's tokens (``spec.extra["side"]``).  The
+    feed-forward may be missing.  ``spec.extra``: ``norm1b``, ``norm2b`` (PartSpecs), ``residual_mult``.
+    Every addition is folded into the norm kernel that next reads the stream (a normed increment
+    beside the plain ones); the last one is handed to the next block."""
+    graph_safe = True
+
+    def __init__(self, env, spec):
+        self.env = env
+        ex = spec.extra
+        self.mult = float(ex.get("residual_mult", 1.0))
+        self.norm1 = build_part("norm", spec.norm1, env)
+        self.mixer = build_part("mixer", spec.mixer, env)
+        self.norm1b = build_part("norm", ex["norm1b"], env)
+        self.children = [("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer),
+                         ("norm1b", self.norm1b, ex["norm1b"])]
+        self.norm2 = self.ffn = self.norm2b = self.side = None
+        if spec.ffn is not None:
+            self.norm2 = build_part("norm", spec.norm2, env)
+            self.ffn = build_part("ffn", spec.ffn, env)
+            self.norm2b = build_part("norm", ex["norm2b"], env)
+            self.children += [("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn),
+                              ("norm2b", self.norm2b, ex["norm2b"])]
+        if ex.get("side") is not None:
+            self.side = build_part("side", ex["side"], env)
+            self.children.append(("side", self.side, ex["side"]))
+        self.children = tuple(self.children)
+        self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
+        self.step_arrays = tuple(sorted({a for _, part, _ in self.children for a in part.step_arrays}))
+
+    def forward(self, h, pending, ctx, cache):
+        state = {"h": h, "pending": pending}
+        for _, stage in self.stages():
+            stage(state, ctx, cache)
+        return state["pending"]
+
+    def stages(self):
+        rest = all(p.graph_safe for p in (self.norm2, self.ffn, self.side) if p is not None)
+        return [(self.norm1.graph_safe, self._stage_norm1), (self.mixer.graph_safe, self._stage_mixer),
+                (rest, self._stage_rest)]
+
+    @staticmethod
+    def _split(h, pending):
+        """(d1, d2, one normed increment or None) of what is still to be added to h."""
+        normed = [p for p in pending if isinstance(p, NormedIncrement)]
+        last = normed.pop() if normed else None
+        d1, d2 = two_increments(h, tuple(p for p in pending if p is not last))
+        return d1, d2, (last.as_arg() if last is not None else None)
+
+    def _stage_norm1(self, state, ctx, cache):
+        h = state["h"]
+        d1, d2, normed = self._split(h, state["pending"])
+        n = ctx.ws.take(tuple(h.shape), self.env.dtype)
+        self.norm1.forward(h, n, d1=d1, d2=d2, normed=normed)
+        state["normed"] = n
+
+    def _stage_mixer(self, state, ctx, cache):
+        state["mixed"] = self.mixer.forward(state.pop("normed"), ctx, cache)
+
+    def _stage_rest(self, state, ctx, cache):
+        h, ws = state["h"], ctx.ws
+        T, d = h.shape
+        pend = (self.norm1b.as_increment(state.pop("mixed"), self.mult),)
+        if self.ffn is not None:
+            n2 = ws.take((T, d), self.env.dtype)
+            proj = self.ffn.input_projection()
+            if proj is not None and self.norm2.can_project(proj):
+                logits = ws.take((T, proj.shape[0]), torch.float32)
+                self.norm2.forward(h, n2, normed=pend[0].as_arg(), proj=proj, proj_out=logits)
+                f = tuple(self.ffn.forward(n2, None, ctx, projected=logits))
+            else:
+                n2_32 = None
+                if self.ffn.wants_f32_input:
+                    n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
+                self.norm2.forward(h, n2, normed=pend[0].as_arg(), out32=None if n2_32 is n2 else n2_32)
+                f = tuple(self.ffn.forward(n2, n2_32, ctx))
+            from ..csrc import hipops
+            for extra in f[1:]:                      # a feed-forward with several results: the norm wants their sum
+                hipops.add_into(f[0], extra[:T])
+            pend = (self.norm2b.as_increment(f[0], self.mult),)
+        if self.side is not None:
+            pend = tuple(self.side.forward(h, pend, ctx))
+        state["pending"] = pend

@@ -9,6 +9,13 @@ logits W_r . x in fp32; the expert with the largest logit (lowest index on ties)
 x is added.  Routed and shared experts run as one grouped product over a row list: group
 e < E holds the tokens routed to expert e, group E every token (at 33 to 64 tokens the shared
 expert's group runs as a plain product of its own over the same rows).
+
+``moe_topk_sigmoid``: router logits in fp32; scores s = sigmoid(logit); the ``top_k`` experts with
+the largest s + bias (a per-expert correction that steers the choice only); each taken expert's
+*output* is weighted with its s (divided by the taken scores' sum if ``renormalize``); a shared
+expert of its own width may run for every token.  The choices of a step are ``top_k`` entries a
+token; the expert plan sorts them by expert, the grouped products walk that list, every entry
+gets an output row of its own and a last kernel forms the weighted sum per token.
 """
 from __future__ import annotations
 
@@ -25,8 +32,12 @@ from ..csrc import hipops
 class DenseGLU(FeedForward):
     graph_safe = True
 
-    def __init__(self, env, hidden_size, intermediate_size):
+    def __init__(self, env, hidden_size, intermediate_size, activation="silu"):
+        """``activation``: the gate's, ``silu`` or ``gelu_tanh``."""
         self.d, self.F = int(hidden_size), int(intermediate_size)
+        if hipops.GATE_ACTS.get(activation, 0) == 0:
+            raise ValueError(f"dense_glu: activation {activation!r} (known: silu, gelu_tanh)")
+        self.activation = activation
         self.w_gate_up = self.w_down = None
 
     def params(self):
@@ -46,7 +57,7 @@ class DenseGLU(FeedForward):
     def forward(self, x, x32, ctx, projected=None):
         T = x.shape[0]
         act = ctx.ws.take((T, self.F), x.dtype)
-        linear(x, self.w_gate_up, act, glu=True, ws=ctx.ws)
+        linear(x, self.w_gate_up, act, glu=self.activation, ws=ctx.ws)
         y = ctx.ws.take((T, self.d), torch.float32)
         linear(act, self.w_down, y, ws=ctx.ws)
         return (y,)
@@ -161,3 +172,88 @@ class MoeTop1Sigmoid(FeedForward):
         linear(x, self.ws_gate_up, act_s, glu=True, ws=ws)
         linear(act_s, self.ws_down, y[T:], ws=ws)
         return (y[:T], y[T:])
+
+
+@register("ffn", "moe_topk_sigmoid")
+class MoeTopKSigmoid(FeedForward):
+    graph_safe = True
+    wants_f32_input = True
+
+    def __init__(self, env, hidden_size, intermediate_size, n_experts, top_k, shared_intermediate_size=None,
+                 score_bias=True, renormalize=False, activation="silu"):
+        self.d, self.F, self.E, self.k = int(hidden_size), int(intermediate_size), int(n_experts), int(top_k)
+        self.Fs = None if shared_intermediate_size is None else int(shared_intermediate_size)
+        if not 1 <= self.k <= self.E or self.E > 512:
+            raise ValueError(f"moe: {self.k} of {self.E} experts (at most 512)")
+        if hipops.GATE_ACTS.get(activation, 0) == 0:
+            raise ValueError(f"moe: activation {activation!r} (known: silu, gelu_tanh)")
+        self.score_bias, self.renormalize, self.activation = bool(score_bias), bool(renormalize), activation
+        self.w_router = self.bias = self.w_gate_up = self.w_down = self.ws_gate_up = self.ws_down = None
+
+    def params(self):
+        d, F, E = self.d, self.F, self.E
+        p = {"router": ParamSpec((E, d), kind="vector")}
+        if self.score_bias:
+            p["correction"] = ParamSpec((E,), kind="vector", init="normal")
+        for e in range(E):
+            p[f"e{e}.gate"], p[f"e{e}.up"], p[f"e{e}.down"] = ParamSpec((F, d)), ParamSpec((F, d)), ParamSpec((d, F))
+        if self.Fs is not None:
+            p["shared.gate"], p["shared.up"] = ParamSpec((self.Fs, d)), ParamSpec((self.Fs, d))
+            p["shared.down"] = ParamSpec((d, self.Fs))
+        return p
+
+    def load(self, t):
+        E = self.E
+        self.w_router = t["router"].contiguous()
+        self.bias = t["correction"].contiguous() if self.score_bias else None
+        dts = {t[f"e{e}.{k}"].dtype for e in range(E) for k in ("gate", "up", "down")}
+        dt = torch.float32 if len(dts) > 1 else dts.pop()
+        gu = torch.stack([torch.cat([t[f"e{e}.gate"].to(dt), t[f"e{e}.up"].to(dt)], dim=0) for e in range(E)])
+        self.w_gate_up = Weight(gu, self.F % 16 == 0)
+        del gu
+        self.w_down = Weight(torch.stack([t[f"e{e}.down"].to(dt) for e in range(E)]))
+        if self.Fs is not None:
+            sdt = t["shared.gate"].dtype if t["shared.gate"].dtype == t["shared.up"].dtype else torch.float32
+            self.ws_gate_up = Weight(torch.cat([t["shared.gate"].to(sdt), t["shared.up"].to(sdt)], dim=0), self.Fs % 16 == 0)
+            self.ws_down = Weight(t["shared.down"])
+
+    def slow_paths(self, page_size):
+        ws = [("experts' gate/up", self.w_gate_up), ("experts' down", self.w_down),
+              ("shared expert's gate/up", self.ws_gate_up), ("shared expert's down", self.ws_down)]
+        return [n for name, w in ws if w is not None for n in w.slow_reason(name)]
+
+    def input_projection(self):
+        return self.w_router if self.w_router is not None and self.w_router.dtype == torch.float32 else None
+
+    def forward(self, x, x32, ctx, projected=None):
+        T, E, F, d, k = x.shape[0], self.E, self.F, self.d, self.k
+        ws = ctx.ws
+        logits = projected
+        if logits is None:
+            logits = ws.take((T, E), torch.float32)
+            hipops.gemm_generic(x32, self.w_router, logits, T, E, d)
+        n = T * k
+        expert, weight = ws.take((n,), torch.int32), ws.take((n,), torch.float32)
+        hipops.router_topk(logits, self.bias, expert, weight, k, renorm=self.renormalize)
+        trace = ctx.extras.get("trace")
+        if trace is not None:                         # a testing aid: which experts each token took, [T, top_k]
+            trace.setdefault("moe_experts", []).append(expert.view(T, k).clone())
+        src, dst, unused = ws.take((n,), torch.int32), ws.take((n,), torch.int32), ws.take((n,), torch.float32)
+        offsets = ws.take((E + 1,), torch.int32)
+        hipops.moe_plan(expert, weight, src, unused, dst, offsets, n, E, False, fan=k)
+        live = min(n, E)
+        # slot s (entries sorted by expert) reads token src[s] and writes the entry's own row dst[s]
+        act = ws.take((n, F), x.dtype)
+        linear(x, self.w_gate_up, act, glu=self.activation, offsets=offsets, n_groups=E, a_rows=src, rows=n, max_rows=T,
+               live_groups=live, ws=ws)
+        y = ws.take((n, d), torch.float32)
+        linear(act, self.w_down, y, offsets=offsets, n_groups=E, y_rows=dst, rows=n, max_rows=T, live_groups=live, ws=ws)
+        ys = None
+        if self.Fs is not None:
+            act_s = ws.take((T, self.Fs), x.dtype)
+            linear(x, self.ws_gate_up, act_s, glu=self.activation, ws=ws)
+            ys = ws.take((T, d), torch.float32)
+            linear(act_s, self.ws_down, ys, ws=ws)
+        out = ws.take((T, d), torch.float32)
+        hipops.moe_combine(y, weight, ys, out, T, k)
+        return (out,)

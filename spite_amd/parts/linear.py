@@ -107,7 +107,8 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
            max_rows=None, tile_shape=0, live_groups=0, ws=None):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
-    With ``glu`` the weight holds gate rows then up rows and y = silu(gate) * up.
+    With ``glu`` the weight holds gate rows then up rows and y = act(gate) * up: ``True`` or
+    ``"silu"``, or ``"gelu_tanh"``.
     ``max_rows``: the most rows that one group can bring (default: ``rows``).
     ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice.
     ``live_groups``: a promise that at most this many groups hold rows (0: none).
@@ -115,11 +116,13 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     tiled = False
     if isinstance(w, Weight):
         w, tiled = w.data, w.tiled
+    glu = hipops.GATE_ACTS[glu]          # True or "silu", "gelu_tanh": the gate's activation
     K = x.shape[-1]
     N = y.shape[-1]
     M = rows if rows is not None else x.shape[0]
     most = max_rows if max_rows is not None else M
-    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0:
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(0) % 8 == 0 \
+            and x.data_ptr() % 16 == 0:
         # few rows: the time is the weights' stream (a very tall matrix, the output table, is
         # streamed faster by the tiled kernel from 33 rows on)
         if most <= SKINNY_MAX_ROWS and not (tiled and most > 32 and offsets is None and N >= 65536):

@@ -23,12 +23,19 @@ class RMSNorm(Norm):
     def load(self, tensors):
         self.weight = tensors["weight"]
 
+    def as_increment(self, y, mult: float):
+        """This norm as the last step of a sublayer's result y on its way into the stream."""
+        from .base import NormedIncrement
+        return NormedIncrement(y, self.weight, float(mult), self.eps)
+
     def can_project(self, proj) -> bool:
         # the kernel keeps the normed row in LDS for the products
         return proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[1] == self.width \
             and hipops.add_rmsnorm_can_project(self.width)
 
-    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, proj=None, proj_out=None):
+    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, proj=None, proj_out=None,
+                normed=None):
+        """``normed``: a ``NormedIncrement``'s (y, weight, mult, eps), added like d1 and d2 after its own norm."""
         hipops.add_rmsnorm(h, self.weight, self.eps, out=out, out32=out32, d1=d1, d2=d2, rows=rows,
                            n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h,
-                           proj=proj, proj_out=proj_out)
+                           proj=proj, proj_out=proj_out, normed=normed)
