@@ -1,0 +1,189 @@
+// Latent attention on the matrix units (bfloat16): query rows [Dk] against cache rows [Dk] of one
+// shared kv head, the value of a key being the first R elements of its row (see latent.hip).
+//
+// Because all heads read the same rows, the heads are the kernel's batch: query row t*H + h is
+// one column of a 16-column MFMA tile, so a decoded token alone fills tiles with its heads, and a
+// prompt's portion fills them with (token, head) pairs.  A workgroup takes up to 128 consecutive
+// query rows of one request (the list `wg`, built on the host from the step's entries: first row
+// and number of rows), one wave per 16 rows.  All waves walk the same blocks of 32 keys, from the
+// first key that the first row may read to the last row's own position; a block is staged once
+// in LDS for all of them: the rows (the S^T = K Q^T operand, in the order of the tiles' rows), and their first R
+// elements transposed (the O^T = V^T P^T operand).  Every row masks by its own position.
+//
+// Tiles: S^T tile tt (of 2) holds the keys (r/4)*8 + tt*4 + r%4 of the block in its rows r, so the
+// eight scores a lane holds are eight consecutive keys: P^T is the next product's operand without a
+// shuffle.  Scores, maximum, sum and the output are fp32.
+#include "common.h"
+
+#define LM_ROWS 128        // query rows per workgroup at most (8 waves of 16)
+#define LM_VT_LD 40        // row stride of the transposed values in LDS (32 keys + 8: no bank conflicts, 16-byte rows)
+
+template <int KQ, int NV>   // Dk <= 32*KQ, R <= 16*NV
+__global__ __launch_bounds__(512)
+void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ kv_pages, bf16* __restrict__ out,
+                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                             const int* __restrict__ block_table, int max_blocks, const int* __restrict__ wg,
+                             int H, int Dk, int R, int ps, int vis, int span, float scale) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int kq = (Dk + 31) >> 5, nv = (R + 15) >> 4;
+    const int ks_ld = kq * 32 + 8;                                  // row stride of the staged rows
+    bf16* Ks = (bf16*)lds_raw;                                      // [32][ks_ld]
+    bf16* Vt = Ks + 32 * ks_ld;                                     // [nv*16][LM_VT_LD]
+    int* kflag = (int*)(Vt + nv * 16 * LM_VT_LD);                   // [32] 1: the key's page was given back
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+    const int c = lane & 15, g4 = lane >> 4;
+    const int row0 = wg[2 * blockIdx.x], nrows = wg[2 * blockIdx.x + 1];
+    const int t_first = row0 / H, t_last = (row0 + nrows - 1) / H;
+    const int* bt = block_table + (size_t)seq_of_token[t_first] * max_blocks;
+    const int key_lo = sp_first_visible(positions[t_first], vis, span), key_hi = positions[t_last];
+
+    // this lane's query row: a column of every tile
+    const int my = wave * 16 + c;
+    const bool row_ok = my < nrows;
+    const int row = row0 + (row_ok ? my : 0);
+    const int my_p = positions[row / H];
+    const int my_lo = sp_first_visible(my_p, vis, span);
+    // what this wave's rows read at all (its first and last row bound it: positions grow with the rows)
+    const int w_first = wave * 16 < nrows ? wave * 16 : 0;
+    const int w_last = wave * 16 + 15 < nrows ? wave * 16 + 15 : nrows - 1;
+    const int wave_lo = sp_first_visible(positions[(row0 + w_first) / H], vis, span);
+    const int wave_hi = wave * 16 < nrows ? positions[(row0 + w_last) / H] : -1;
+
+    bf16x8 qf[KQ];
+#pragma unroll
+    for (int k = 0; k < KQ; ++k) {
+        const int f = k * 32 + g4 * 8;
+        bf16x8 z;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) z[e] = (bf16)0.f;
+        qf[k] = (k < kq && f < Dk) ? *(const bf16x8*)(q + (size_t)row * Dk + f) : z;
+    }
+    // the staged rows' elements past Dk are zero for good
+    for (int i = tid; i < 32 * (ks_ld - Dk); i += nthreads) {
+        const int key = i / (ks_ld - Dk), f = Dk + i % (ks_ld - Dk);
+        Ks[key * ks_ld + f] = (bf16)0.f;
+    }
+    for (int i = tid; i < (nv * 16 - R) * LM_VT_LD; i += nthreads) Vt[R * LM_VT_LD + i] = (bf16)0.f;
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 o[NV];
+#pragma unroll
+    for (int a = 0; a < NV; ++a) o[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int chunks = Dk >> 3;                                     // 16-byte pieces of a row
+
+    for (int blk0 = key_lo & ~31; blk0 <= key_hi; blk0 += 32) {
+        __syncthreads();                                            // the last block's readers are done
+        for (int i = tid; i < 32 * chunks; i += nthreads) {
+            const int key = i / chunks, f = (i - key * chunks) << 3;
+            const int j = blk0 + key;
+            bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (bf16)0.f;
+            int gone = 0;
+            if (j >= key_lo && j <= key_hi) {
+                const int page = bt[j / ps];
+                if (page >= 0) v = *(const bf16x8*)(kv_pages + ((size_t)page * ps + j % ps) * Dk + f);
+                else gone = 1;
+            }
+            // LDS row of a key: the 16 rows of S^T tile tt lie together, tile row (key/8)*4 + key%4
+            *(bf16x8*)(Ks + ((((key >> 2) & 1) << 4) + ((key >> 3) << 2) + (key & 3)) * ks_ld + f) = v;
+            if (f < R) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) Vt[(f + e) * LM_VT_LD + key] = v[e];
+            }
+            if (f == 0) kflag[key] = gone;
+        }
+        __syncthreads();
+        if (blk0 + 31 < wave_lo || blk0 > wave_hi) continue;        // nothing here for this wave's rows
+
+        f32x4 s[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const bf16* kr = Ks + (tt * 16 + c) * ks_ld + g4 * 8;
+#pragma unroll
+            for (int k = 0; k < KQ; ++k)
+                if (k < kq) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kr + k * 32), qf[k], s[tt], 0, 0, 0);
+        }
+        float mx = -INFINITY;
+        bool ok[2][4];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = g4 * 8 + tt * 4 + i, j = blk0 + key;
+                ok[tt][i] = row_ok && j >= my_lo && j <= my_p;
+                const float v = ok[tt][i] ? (kflag[key] ? NAN : s[tt][i] * scale) : -INFINITY;
+                s[tt][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = rows4_max(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+        float sum = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = ok[tt][i] ? __expf(s[tt][i] - m_new) : 0.f;
+                sum += e;
+                pf[tt * 4 + i] = (bf16)e;
+            }
+        sum = rows4_sum(sum);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int a = 0; a < NV; ++a) {
+            if (a < nv) {
+                o[a] = o[a] * alpha;
+                o[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(Vt + (a * 16 + c) * LM_VT_LD + g4 * 8), pf, o[a], 0, 0, 0);
+            }
+        }
+    }
+    if (!row_ok) return;
+    // o[a][i] of lane (c, g4) is O[row c][a*16 + g4*4 + i]
+    const float inv = 1.0f / fmaxf(l_run, 1e-30f);
+    bf16* orow = out + (size_t)row * R;
+#pragma unroll
+    for (int a = 0; a < NV; ++a) {
+        const int col = a * 16 + g4 * 4;
+        if (a < nv && col < R) {
+            bf16x4 w;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = (bf16)(o[a][i] * inv);
+            *(bf16x4*)(orow + col) = w;
+        }
+    }
+}
+
+// `wg`: int32 pairs (first query row, rows <= 128) on the device, `n_wg` of them, each within one
+// request's rows of the step; `max_rows`: the most rows of any pair (it sizes the workgroups).
+extern "C" int spite_attn_latent_mfma(const void* q, const void* kv_pages, void* out, const int* positions,
+                                      const int* seq_of_token, const int* block_table, int max_blocks, const int* wg,
+                                      int n_wg, int max_rows, int H, int Dk, int R, int page_size, int vis, int span,
+                                      float scale, hipStream_t st) {
+    SP_REQUIRE(H > 0 && n_wg >= 0 && max_rows >= 0 && max_rows <= LM_ROWS, "latent attention: %d rows a workgroup, at most %d", max_rows, LM_ROWS);
+    SP_REQUIRE(Dk > 0 && Dk % 8 == 0 && R > 0 && R % 8 == 0 && R <= Dk && Dk <= 576 && R <= 512,
+               "latent attention (MFMA): rows of %d with a latent of %d: multiples of 8, at most 576 and 512", Dk, R);
+    SP_REQUIRE(page_size > 0 && max_blocks > 0, "latent attention: bad page size %d or table width %d", page_size, max_blocks);
+    SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "latent attention: chunk or window of %d", span);
+    SP_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kv_pages & 15) == 0 && ((uintptr_t)out & 7) == 0, "latent attention: operands must be 16-byte aligned");
+    if (n_wg == 0 || max_rows == 0) return 0;
+    const int kq = (Dk + 31) / 32, nv = (R + 15) / 16;
+    const int nw = (max_rows + 15) / 16;
+    const size_t sh = ((size_t)32 * (kq * 32 + 8) + (size_t)nv * 16 * LM_VT_LD) * sizeof(bf16) + 32 * sizeof(int);
+#define SP_LM(KQV, NVV) do { \
+        auto kern = attn_latent_mfma_kernel<KQV, NVV>; \
+        static bool allowed = false; \
+        if (sh > 48 * 1024 && !allowed) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
+            if (e != hipSuccess) return sp_fail("latent attention: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e)); allowed = true; } \
+        kern<<<n_wg, nw * 64, sh, st>>>((const bf16*)q, (const bf16*)kv_pages, (bf16*)out, positions, seq_of_token, \
+                                        block_table, max_blocks, wg, H, Dk, R, page_size, vis, span, scale); } while (0)
+    if (kq <= 6 && nv <= 8) SP_LM(6, 8);
+    else if (kq <= 10 && nv <= 16) SP_LM(10, 16);
+    else SP_LM(18, 32);
+#undef SP_LM
+    SP_LAUNCH_CHECK("attn_latent_mfma");
+    return 0;
+}

@@ -59,6 +59,7 @@ def lib():
             "spite_mfma_loop": [P, I, I, F, P],
             "spite_latent_prepare": [P, I, P, I, P, P, I, P, P, P, P, F, I, I, I, I, I, I, I, P, P, P],
             "spite_attn_latent_generic": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
+            "spite_attn_latent_mfma": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, F, P],
             "spite_router_topk": [P, P, P, P, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
@@ -687,6 +688,40 @@ def gated_rows(a, ids, table, col0, g):
                                   _stream()), "gated_rows")
 
 
+LATENT_WG_ROWS = 128      # query rows that one workgroup of the MFMA kernel takes at most
+
+
 def attn_latent_mfma_ok(Dk, R, page_size) -> bool:
     """Whether the MFMA kernel of latent attention takes rows of Dk with a latent of R (bfloat16)."""
-    return False
+    return Dk % 8 == 0 and R % 8 == 0 and 0 < R <= 512 and R <= Dk <= 576
+
+
+def latent_workgroups(counts, cu_seqlens, H):
+    """The MFMA kernel's work list for a step: int32 pairs (first query row, rows), at most
+    ``LATENT_WG_ROWS`` rows each and every pair inside one entry's rows (entry i holds the query rows
+    cu[i]*H .. cu[i+1]*H), flat; and (pairs, the most rows of a pair)."""
+    out = []
+    most = 0
+    for i, n in enumerate(counts):
+        rows, r0 = int(n) * H, int(cu_seqlens[i]) * H
+        for off in range(0, rows, LATENT_WG_ROWS):
+            k = min(LATENT_WG_ROWS, rows - off)
+            out += [r0 + off, k]
+            most = max(most, k)
+    return np.asarray(out, dtype=np.int32), (len(out) // 2, most)
+
+
+def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg, n_wg, max_rows, T, H, Dk, R, vis, span, scale):
+    """As ``attn_latent_generic`` on the matrix units (bfloat16; see ``attn_latent_mfma_ok``).  ``wg``:
+    the work list of ``latent_workgroups`` on the device."""
+    _latent_checks(q, kv_pages, out, positions, seq_of_token, block_table, T, H, Dk, R, "latent attention (MFMA)")
+    if q.dtype != torch.bfloat16:
+        raise KernelError(f"latent attention (MFMA): bfloat16 only, got {q.dtype}")
+    if wg.numel() < 2 * n_wg or max_rows > LATENT_WG_ROWS:
+        raise KernelError("latent attention (MFMA): work list too short or its pairs too long")
+    dt = torch.bfloat16
+    _check(lib().spite_attn_latent_mfma(
+        _ptr(q, "q", dt), _ptr(kv_pages, "kv_pages", dt), _ptr(out, "out", dt), _ptr(positions, "positions", torch.int32),
+        _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
+        block_table.shape[1], _ptr(wg, "wg", torch.int32), int(n_wg), int(max_rows), H, Dk, R, kv_pages.shape[2],
+        VIS[vis], int(span or 0), float(scale), _stream()), "latent attention (MFMA)")

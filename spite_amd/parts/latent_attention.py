@@ -19,9 +19,17 @@ from __future__ import annotations
 
 import torch
 
-from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, build as build_part
+from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, register_step_array, build as build_part
 from .linear import linear, Weight
 from ..csrc import hipops
+
+
+def _workgroups_name(H: int) -> str:
+    """The step array with the MFMA kernel's work list for models of H heads (registered on demand:
+    the list depends on the step's entries and on H alone)."""
+    name = f"latent_attention.workgroups/{H}"
+    register_step_array(name, lambda host: hipops.latent_workgroups(host.counts, host.cu_seqlens, H))
+    return name
 
 
 @register("mixer", "latent_attention")
@@ -57,6 +65,9 @@ class LatentAttention(Mixer):
         if self.rot_dims > self.r:
             raise ValueError(f"latent attention: {self.rot_dims} turning elements of a rotated part of {self.r}")
         self.wq = self.wdkv = self.w_norm = self.w_absorb = self.w_up = self.wo = None
+        self.mfma = env.dtype == torch.bfloat16 and hipops.attn_latent_mfma_ok(self.Dk, self.R, 0)
+        self._wg = _workgroups_name(self.H) if self.mfma else None
+        self.step_arrays = (self._wg,) if self.mfma else ()
 
     def params(self):
         d, H, n, r, v, R = self.d, self.H, self.n, self.r, self.v, self.R
@@ -74,7 +85,8 @@ class LatentAttention(Mixer):
             self.wdkv = Weight(t["dkv"])
             self.w_norm = t["dkv.norm"].contiguous()
         # U_h^T as a product's weight [out = R, in = n]; V_h is one already: [out = v, in = R]
-        self.w_absorb = Weight(t["uk"].view(H, n, R).transpose(1, 2).contiguous())
+        # (its input rows are column ranges of the query rows: operand order only if those stay aligned)
+        self.w_absorb = Weight(t["uk"].view(H, n, R).transpose(1, 2).contiguous(), (n + self.r) % 8 == 0)
         self.w_up = Weight(t["uv"].view(H, v, R))
         self.wo = Weight(t["o"])
 
@@ -116,9 +128,10 @@ class LatentAttention(Mixer):
         linear(q.view(T * H, n + r)[:, :n], self.w_absorb, qa[:, :R], offsets=offsets_h, n_groups=H, a_rows=rows_th,
                y_rows=rows_th, rows=H * T, max_rows=T, ws=ws)
         o_lat = ws.take((T * H, R), x.dtype)
-        if x.dtype == torch.bfloat16 and hipops.attn_latent_mfma_ok(Dk, R, cache.page_size):
+        if self.mfma:
+            wg, (n_wg, most) = ctx.derived[self._wg]
             hipops.attn_latent_mfma(qa, cache.k_pages, o_lat, ctx.positions, ctx.seq_of_token, cache.block_table,
-                                    T, H, Dk, R, self.visibility, self.span, self.scale)
+                                    wg, n_wg, most, T, H, Dk, R, self.visibility, self.span, self.scale)
         else:
             hipops.attn_latent_generic(qa, cache.k_pages, o_lat, ctx.positions, ctx.seq_of_token, cache.block_table,
                                        T, H, Dk, R, self.visibility, self.span, self.scale)

@@ -1,0 +1,448 @@
+"""The Ravenex design in the engine against the plain implementation (``plain_ravenex``): every
+mechanism's kernel alone, whole prompts, decoding through the cache, portions down to two tokens,
+mixed batches with pages and slots used again, window edges, far keys, generation."""
+from __future__ import annotations
+
+import copy
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_ravenex as plain
+
+
+def _mixer(heads, dim, rot, vdim, rank, window, kv_from=None, base=10000.0, scale=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "rot": {"base": base, "dims": rot},
+         "scale": scale if scale is not None else 1.0 / math.sqrt(dim + rot)}
+    if window is not None:
+        m["mask"] = {"size": window}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def _moe(experts, top, ff, shared):
+    m = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}}
+    if shared is not None:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def _layer(mixer, mlp):
+    return {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+
+
+# sizes that no fast kernel takes (odd widths, heads and ranks); windows of readers below and above
+# their cache's owner, a layer without a feed-forward, one expert a token, no shared expert
+SMALL = {"architecture": "Ravenex", "vocab": 96, "width": 40, "residual_mult": 0.6, "norm": {"eps": 1e-5},
+         "token_side": {"dim": 6},
+         "layers": [_layer(_mixer(3, 12, 6, 10, 20, 9), {"kind": "dense", "ff": 56}),
+                    _layer(_mixer(4, 10, 6, 8, 20, 5, kv_from=0), _moe(5, 2, 24, 16)),
+                    _layer(_mixer(2, 8, 4, 12, 12, None, base=500.0), None),
+                    _layer(_mixer(2, 6, 4, 6, 12, 7, kv_from=2, base=500.0), _moe(4, 1, 16, None)),
+                    _layer(_mixer(3, 12, 6, 10, 20, 13, kv_from=0), {"kind": "dense", "ff": 24})]}
+# sizes that the matrix-unit kernels take in bfloat16; more heads than a tile has columns
+WIDE = {"architecture": "Ravenex", "vocab": 320, "width": 128, "residual_mult": 0.8, "norm": {"eps": 1e-6},
+        "token_side": {"dim": 8},
+        "layers": [_layer(_mixer(4, 32, 16, 32, 64, 40), {"kind": "dense", "ff": 128}),
+                   _layer(_mixer(20, 32, 16, 16, 64, 40, kv_from=0), _moe(6, 3, 32, 48)),
+                   _layer(_mixer(4, 64, 32, 32, 96, None, base=1000.0), _moe(6, 2, 64, None)),
+                   _layer(_mixer(6, 64, 32, 48, 96, 33, kv_from=2, base=1000.0), {"kind": "dense", "ff": 64})]}
+# no token side input
+BARE = dict(copy.deepcopy(SMALL), token_side=None)
+CONFIGS = {"small": SMALL, "wide": WIDE, "bare": BARE}
+PAGE = {"small": 16, "wide": 32, "bare": 8}
+
+
+def planted(cfg, seed, qk_gain=3.0, router_gain=8.0, std=0.08):
+    """Random tensors with queries, down-projections and routers scaled up: attention far from
+    uniform, experts clearly apart, so a wrong key or expert moves the logits."""
+    from spite_amd.weights.random_init import random_tensors
+    t = random_tensors(cfg, seed, std)
+    for name in list(t):
+        if name.endswith(".mix.q") or name.endswith(".mix.dkv"):
+            t[name] = t[name] * qk_gain
+        if name.endswith(".mlp.router"):
+            t[name] = t[name] * router_gain
+        if name.endswith(".mlp.correction"):
+            t[name] = t[name] * 2.0
+    return t
+
+
+def make_model(folder, cfg, seed, dtype, **kw):
+    from spite_amd.weights.random_init import write_random_model
+    write_random_model(str(folder), cfg, seed, dtype=dtype, overrides=planted(cfg, seed, **kw))
+    return H.read_weights(str(folder))
+
+
+def requests(vocab, lengths, seed):
+    return {f"r{i}": H.random_tokens(vocab, n, seed + 13 * i) for i, n in enumerate(lengths)}
+
+
+def plain_rows(cfg, weights, reqs, experts=None):
+    rows = {}
+    for rid, toks in reqs.items():
+        out = plain.forward(cfg, weights, toks, experts=None if experts is None else experts[rid]).to(torch.float32).numpy()
+        for i in range(len(toks)):
+            rows[(rid, i)] = out[i]
+    return rows
+
+
+def engine(folder, dtype, name, **kw):
+    from spite_amd import Engine
+    kw.setdefault("page_size", PAGE[name])
+    kw.setdefault("cache_tokens", 1024)
+    kw.setdefault("max_requests", 4)
+    return Engine(str(folder), dtype=dtype, device="cuda:0", **kw)
+
+
+def poison(eng):
+    """Every cache row holds NaN until it is written: a row read before that shows in the logits."""
+    for g in eng.cache.groups:
+        for half in g.halves():
+            if half is not None and half.numel():
+                half.fill_(float("nan"))
+
+
+def scale_of(rows):
+    return max(float(np.abs(v).max()) for v in rows.values())
+
+
+# ------------------------------------------------------------------------------------------ without a GPU
+def test_registry_and_tensor_names():
+    from spite_amd.config import read_config, RavenexConfig
+    from spite_amd.engine.model import Model
+    from spite_amd.engine.context import Env
+    arch, cfg = read_config(SMALL)
+    assert arch.name == "Ravenex" and isinstance(cfg, RavenexConfig)
+    assert cfg.layers[1].mixer.kv_from == 0 and cfg.layers[2].mixer.window is None and cfg.layers[2].mlp is None
+    model = Model(arch.build_spec(cfg), Env(torch.float32, torch.device("cpu")))
+    names = {n for n, _, _, _ in model.tensor_plan()}
+    assert {"embed", "side.embed", "final.norm", "head", "l0.mix.dkv", "l0.mix.dkv.norm", "l1.mlp.e4.down", "l1.mlp.correction",
+            "l1.mlp.shared.up", "l3.mlp.router", "l4.side.proj", "l0.norm2b"} <= names
+    assert "l1.mix.dkv" not in names and "l2.norm2" not in names and "l3.mlp.shared.up" not in names
+    needs = model.cache_needs()
+    # the cache of layer 0 keeps what its widest reader needs; the one of layer 2 everything
+    assert needs[0].kv.visibility == "window" and needs[0].kv.span == 13 and needs[0].kv.head_dim == 26
+    assert needs[2].kv.visibility == "full" and needs[1] is None and len(needs) == 3
+    assert not any(n.startswith("side.") or ".side." in n for n, _, _, _ in
+                   Model(arch.build_spec(read_config(BARE)[1]), Env(torch.float32, torch.device("cpu"))).tensor_plan())
+
+
+def test_config_errors_are_collected():
+    from spite_amd.config import read_config, ConfigError
+    bad = copy.deepcopy(SMALL)
+    del bad["width"]
+    bad["layers"][1]["mixer"]["kv_from"] = 3
+    bad["layers"][3]["mlp"]["router"]["top"] = 9
+    bad["layers"][0]["type"] = "other"
+    with pytest.raises(ConfigError) as e:
+        read_config(bad)
+    msg = str(e.value)
+    assert "width" in msg and "kv_from" in msg and "top" in msg and "type" in msg
+
+
+def test_plain_window_and_rotation():
+    ok = plain.window_mask(6, 3)
+    assert ok[5].tolist() == [False, False, False, True, True, True] and ok[1].tolist() == [True, True] + [False] * 4
+    x = torch.arange(8, dtype=torch.float64).view(1, 8)
+    y = plain.rotate_adjacent(x, torch.tensor([0]), 100.0, 4)
+    assert torch.equal(x, y)                                       # position 0 turns nothing
+    y = plain.rotate_adjacent(x, torch.tensor([3]), 100.0, 4)
+    a = 3.0                                                        # pair 0 turns by p * 1
+    assert abs(float(y[0, 0]) - (0 * math.cos(a) - 1 * math.sin(a))) < 1e-12 and torch.equal(y[0, 4:], x[0, 4:])
+    assert abs(float(y[0, 3]) - (3 * math.cos(0.3) + 2 * math.sin(0.3))) < 1e-12     # pair 1: 100^(-2/4) = 0.1
+
+
+# ------------------------------------------------------------------------------------------ kernels alone
+@pytest.mark.gpu
+@pytest.mark.parametrize("E,top,bias", [(5, 2, True), (70, 3, True), (4, 1, False), (6, 6, True)])
+def test_router_topk_kernel(E, top, bias):
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(E + top)
+    T = 37
+    logits = torch.randn(T, E, generator=g) * 3
+    logits[3, :] = 0.25                                            # all equal: the lowest indices win
+    corr = torch.randn(E, generator=g) if bias else torch.zeros(E)
+    # the logits are the plain router's products with a unit matrix
+    idx, wt = plain.router_choice(logits.double(), torch.eye(E, dtype=torch.float64), corr.double(), top)
+    dev = "cuda:0"
+    expert = torch.empty(T * top, dtype=torch.int32, device=dev)
+    weight = torch.empty(T * top, dtype=torch.float32, device=dev)
+    hipops.router_topk(logits.to(dev), corr.to(dev) if bias else None, expert, weight, top)
+    assert torch.equal(expert.cpu().view(T, top).long(), idx)
+    assert torch.allclose(weight.cpu().view(T, top).double(), wt, atol=1e-6)
+    if not bias:
+        assert expert.cpu().view(T, top)[3].tolist() == list(range(top))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,M,N,K", [("float32", 9, 24, 40), ("bfloat16", 5, 64, 128), ("bfloat16", 100, 64, 128),
+                                         ("bfloat16", 200, 48, 72), ("bfloat16", 7, 20, 40)])
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_gated_products_activation(dtype, M, N, K, act):
+    from spite_amd.parts.linear import linear, Weight
+    dt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(M + N)
+    x = (torch.randn(M, K, generator=g)).to(dt)
+    w = (torch.randn(2 * N, K, generator=g) / math.sqrt(K) * 2).to(dt)
+    y = torch.empty(M, N, dtype=dt, device="cuda:0")
+    linear(x.cuda(), Weight(w.cuda(), N % 16 == 0), y, glu=act)
+    z = x.double() @ w.double().T
+    want = (plain.silu if act == "silu" else plain.gelu_tanh)(z[:, :N]) * z[:, N:]
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert float((y.cpu().double() - want).abs().max()) <= tol * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d", [40, 128, 333])
+def test_norm_with_normed_increment(d):
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(d)
+    T = 11
+    h, y, d1 = (torch.randn(T, d, generator=g) for _ in range(3))
+    wn, w = torch.rand(d, generator=g) + 0.5, torch.rand(d, generator=g) + 0.5
+    hd, out = h.cuda().clone(), torch.empty(T, d, device="cuda:0")
+    hipops.add_rmsnorm(hd, w.cuda(), 1e-5, out=out, d1=d1.cuda(), normed=(y.cuda(), wn.cuda(), 0.7, 1e-3))
+    want_h = h.double() + d1.double() + 0.7 * plain.norm(y.double(), wn.double(), 1e-3)
+    assert torch.allclose(hd.cpu().double(), want_h, atol=1e-5)
+    assert torch.allclose(out.cpu().double(), plain.norm(want_h, w.double(), 1e-5), atol=1e-5)
+    # the stream itself as output, in bfloat16, and a call that only adds
+    hd2, cast = h.cuda().clone(), torch.empty(T, d, device="cuda:0", dtype=torch.bfloat16)
+    hipops.add_rmsnorm(hd2, None, 1e-5, out=cast, normed=(y.cuda(), wn.cuda(), 0.7, 1e-3), plain_out=True)
+    hd3 = h.cuda().clone()
+    hipops.add_rmsnorm(hd3, None, 1e-5, normed=(y.cuda(), wn.cuda(), 0.7, 1e-3))
+    assert torch.equal(hd2, hd3) and torch.equal(cast, hd2.to(torch.bfloat16))
+
+
+def _attention_case(Hh, Dk, R, ps, lens_new, starts, vis, span, dtype, seed):
+    """Query rows and a paged cache for requests with ``starts`` cached positions and ``lens_new`` new
+    tokens; pages dealt out of order.  Returns the kernels' arguments and the plain result."""
+    g = torch.Generator().manual_seed(seed)
+    dt = getattr(torch, dtype)
+    n = len(starts)
+    totals = [s + c for s, c in zip(starts, lens_new)]
+    n_pages = sum(-(-t // ps) for t in totals) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = max(-(-t // ps) for t in totals) + 1
+    table = torch.full((n, width), -1, dtype=torch.int32)
+    pages = torch.full((n_pages, 1, ps, Dk), float("nan"))
+    rows_of = []
+    for i, t in enumerate(totals):
+        kv = torch.randn(t, Dk, generator=g).to(dt).float()
+        rows_of.append(kv)
+        for b in range(-(-t // ps)):
+            pg = perm.pop()
+            table[i, b] = pg
+            chunk = kv[b * ps:(b + 1) * ps]
+            pages[pg, 0, :chunk.shape[0]] = chunk
+    T = sum(lens_new)
+    q = (torch.randn(T * Hh, Dk, generator=g) * 1.5).to(dt).float()
+    positions = torch.tensor([s + j for s, c in zip(starts, lens_new) for j in range(c)], dtype=torch.int32)
+    seq = torch.tensor([i for i, c in enumerate(lens_new) for _ in range(c)], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(Dk)
+    want = torch.zeros(T * Hh, R, dtype=torch.float64)
+    for t in range(T):
+        p, kv = int(positions[t]), rows_of[int(seq[t])].double()
+        lo = 0 if vis == "full" else max(0, p - span + 1)
+        for h in range(Hh):
+            s = (kv[lo:p + 1] @ q[t * Hh + h].double()) * scale
+            want[t * Hh + h] = torch.softmax(s, 0) @ kv[lo:p + 1, :R]
+    dev = "cuda:0"
+    cu = np.concatenate([[0], np.cumsum(lens_new)])
+    return dict(q=q.to(dt).to(dev), pages=pages.to(dt).to(dev), positions=positions.to(dev), seq=seq.to(dev),
+                table=table.to(dev), T=T, scale=scale, want=want, counts=np.asarray(lens_new), cu=cu)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("Hh,Dk,R,ps,vis,span", [(3, 26, 20, 8, "window", 9), (2, 16, 12, 16, "full", 0), (5, 40, 24, 4, "window", 33)])
+def test_latent_attention_plain_kernel(Hh, Dk, R, ps, vis, span):
+    from spite_amd.csrc import hipops
+    c = _attention_case(Hh, Dk, R, ps, [1, 17, 40, 1, 2], [50, 0, 23, 0, 31], vis, span, "float32", Dk)
+    out = torch.empty(c["T"] * Hh, R, device="cuda:0")
+    hipops.attn_latent_generic(c["q"], c["pages"], out, c["positions"], c["seq"], c["table"], c["T"], Hh, Dk, R, vis, span, c["scale"])
+    assert float((out.cpu().double() - c["want"]).abs().max()) < 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("Hh,Dk,R,ps,vis,span", [(6, 128, 96, 64, "window", 72), (20, 80, 64, 32, "window", 40), (3, 48, 40, 16, "full", 0),
+                                                 (130, 96, 64, 32, "window", 5), (16, 192, 128, 8, "full", 0), (4, 320, 256, 32, "window", 100),
+                                                 (2, 576, 512, 64, "full", 0)])
+def test_latent_attention_matrix_kernel(Hh, Dk, R, ps, vis, span):
+    """Single tokens beside portions, windows that end inside a block of keys, more query rows than a
+    workgroup takes, rows of one token in two workgroups, every pair of template sizes."""
+    from spite_amd.csrc import hipops
+    assert hipops.attn_latent_mfma_ok(Dk, R, ps)
+    c = _attention_case(Hh, Dk, R, ps, [1, 37, 1, 70, 2], [199, 0, 0, 45, 63], vis, span, "bfloat16", Dk + Hh)
+    wg, (n_wg, most) = hipops.latent_workgroups(c["counts"], c["cu"], Hh)
+    assert most <= hipops.LATENT_WG_ROWS and int(wg[1::2].sum()) == c["T"] * Hh
+    out = torch.full((c["T"] * Hh, R), float("nan"), device="cuda:0", dtype=torch.bfloat16)
+    hipops.attn_latent_mfma(c["q"], c["pages"], out, c["positions"], c["seq"], c["table"], torch.from_numpy(wg).cuda(), n_wg, most,
+                            c["T"], Hh, Dk, R, vis, span, c["scale"])
+    ref = torch.empty_like(out)
+    hipops.attn_latent_generic(c["q"], c["pages"], ref, c["positions"], c["seq"], c["table"], c["T"], Hh, Dk, R, vis, span, c["scale"])
+    tol = 0.02 * float(c["want"].abs().max())
+    assert float((out.cpu().double() - c["want"]).abs().max()) < tol
+    assert float((ref.cpu().double() - c["want"]).abs().max()) < tol
+
+
+# ------------------------------------------------------------------------------------------ the model in the engine
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            folder = tmp_path_factory.mktemp(f"ravenex_{name}_{dtype}")
+            # milder weights for the 16-bit runs: with very sharp attention the rounding of a score moves the logits
+            # by more than any tolerance that would still tell a wrong key
+            kw = {} if dtype == "float32" else dict(qk_gain=1.5, router_gain=4.0, std=0.05)
+            made[(name, dtype)] = (folder, make_model(folder, CONFIGS[name], seed=11 + len(name), dtype=dtype, **kw))
+        return made[(name, dtype)]
+    return get
+
+
+LENGTHS = {"small": [1, 45, 23, 60, 2, 31, 17], "wide": [90, 1, 140, 33, 75], "bare": [30, 1, 44, 9]}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["small", "wide", "bare"])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_float32_against_plain(models, name, schedule):
+    """True 32-bit: every schedule gives the plain implementation's logits at every position.  The
+    pools start poisoned and are small: pages and slots are used again in the mixed schedule."""
+    cfg = CONFIGS[name]
+    folder, weights = models(name, "float32")
+    reqs = requests(cfg["vocab"], LENGTHS[name], 5)
+    ref = plain_rows(cfg, weights, reqs)
+    steps = {"whole": H.schedule_whole, "tail": lambda r: H.schedule_tail_one_by_one(r, tail=28),
+             "portions": H.schedule_portions, "mixed": lambda r: H.schedule_mixed(r, seed=3, max_live=4)}[schedule](reqs)
+    eng = engine(folder, "float32", name, cache_tokens=4 * (max(LENGTHS[name]) + PAGE[name]))
+    poison(eng)
+    got = H.collect(steps, H.run_trace_inprocess(eng, steps), cfg["vocab"])
+    err, where = H.max_diff(got, ref)
+    assert err <= 2e-4 * scale_of(ref), f"{err} at {where} (scale {scale_of(ref)})"
+    assert all(eng.cache.free_pages(g) == eng.cache.total_pages(g) for g in range(eng.cache.n_groups()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["small", "wide"])
+def test_bfloat16_against_plain_and_itself(models, name):
+    """bfloat16 through the serving kernels: whole prompts against the plain implementation (which
+    follows the engine's experts, two scores being tied at this precision now and then), then the
+    other schedules against the whole prompts."""
+    cfg = CONFIGS[name]
+    folder, weights = models(name, "bfloat16")
+    reqs = requests(cfg["vocab"], LENGTHS[name], 8)
+    eng = engine(folder, "bfloat16", name, cache_tokens=4 * (max(LENGTHS[name]) + PAGE[name]))
+    if name == "wide":
+        assert not eng.slow_paths, eng.slow_paths
+    poison(eng)
+    whole = H.schedule_whole(reqs)
+    routing = {}
+    rows = H.collect(whole, H.run_trace_inprocess(eng, whole, routing), cfg["vocab"])
+    moe = [i for i, L in enumerate(cfg["layers"]) if L["mlp"] and L["mlp"]["kind"] == "moe"]
+    experts = {rec["entries"][0]["id"]: {L: torch.from_numpy(routing[rec["step"]][k]).long() for k, L in enumerate(moe)} for rec in whole}
+    ref = plain_rows(cfg, weights, reqs, experts)
+    scale = scale_of(ref)
+    err, where = H.max_diff(rows, ref)
+    assert err <= 0.05 * scale, f"{err} at {where} (scale {scale})"
+    for steps in (H.schedule_tail_one_by_one(reqs, tail=28), H.schedule_portions(reqs), H.schedule_mixed(reqs, seed=4, max_live=4)):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), cfg["vocab"])
+        err, where = H.max_diff(got, rows)
+        assert err <= 0.05 * scale, f"{err} at {where} (scale {scale})"
+
+
+def _one_layer(window, heads=3, wide=False):
+    mix = _mixer(4, 32, 16, 32, 64, window) if wide else _mixer(heads, 12, 6, 10, 20, window)
+    return {"architecture": "Ravenex", "vocab": 64, "width": 128 if wide else 40, "residual_mult": 1.0, "norm": {"eps": 1e-5},
+            "token_side": {"dim": 4}, "layers": [_layer(mix, {"kind": "dense", "ff": 32})]}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,wide", [("float32", False), ("bfloat16", True)])
+@pytest.mark.parametrize("decoded", [False, True])
+def test_window_edges(tmp_path, dtype, wide, decoded):
+    """One layer, a window of 11 over pages of 8: the logits at position i do not
+    move at all when the token just outside the window changes, and move when the one just inside
+    does; in a prompt and when the positions are decoded one by one."""
+    W = 11
+    cfg = _one_layer(W, wide=wide)
+    make_model(tmp_path, cfg, seed=2, dtype=dtype, qk_gain=3.0)
+    from spite_amd import Engine
+    eng = Engine(str(tmp_path), dtype=dtype, page_size=8, cache_tokens=256, max_requests=2, device="cuda:0")
+    base = H.random_tokens(64, 48, 1)
+
+    def run(toks):
+        reqs = {"a": toks}
+        steps = H.schedule_tail_one_by_one(reqs, tail=30) if decoded else H.schedule_whole(reqs)
+        return H.collect(steps, H.run_trace_inprocess(eng, steps), 64)
+    ref = run(base)
+    for i in (20, 31, 47):
+        outside, inside = list(base), list(base)
+        outside[i - W] = (base[i - W] + 7) % 64
+        inside[i - W + 1] = (base[i - W + 1] + 7) % 64
+        a, b = run(outside)[("a", i)], run(inside)[("a", i)]
+        assert np.array_equal(a, ref[("a", i)]), f"position {i} sees the token {W} back"
+        assert float(np.abs(b - ref[("a", i)]).max()) > 1e-4 * float(np.abs(ref[("a", i)]).max()), f"position {i} misses the window's first token"
+
+
+@pytest.mark.gpu
+def test_far_keys_and_long_decoding(tmp_path):
+    """Every earlier key is read (no window), attention is sharp, the prompt spans many small pages
+    and more than a hundred tokens are decoded one by one: a lost key anywhere shows against the
+    plain implementation."""
+    cfg = _one_layer(None)
+    weights = make_model(tmp_path, cfg, seed=4, dtype="float32", qk_gain=6.0)
+    from spite_amd import Engine
+    eng = Engine(str(tmp_path), dtype="float32", page_size=8, cache_tokens=512, max_requests=2, device="cuda:0")
+    poison(eng)
+    reqs = {"a": H.random_tokens(64, 330, 6)}
+    ref = plain_rows(cfg, weights, reqs)
+    steps = H.schedule_tail_one_by_one(reqs, tail=130)
+    got = H.collect(steps, H.run_trace_inprocess(eng, steps), 64)
+    err, where = H.max_diff(got, ref)
+    assert err <= 2e-4 * scale_of(ref), f"{err} at {where}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["small", "wide"])
+def test_greedy_generation(models, name):
+    """Through the engine's own entry point and scheduler: prompts of unequal length, more new tokens
+    than the windows are long, in true 32-bit: the plain implementation's greedy tokens."""
+    cfg = CONFIGS[name]
+    folder, weights = models(name, "float32")
+    prompts = [H.random_tokens(cfg["vocab"], n, 40 + n) for n in (1, 19, 7)]
+    eng = engine(folder, "float32", name, cache_tokens=512, max_batch_tokens=16)
+    n_new = 50 if name == "small" else 12
+    got = eng.generate(prompts, max_tokens=n_new, temperature=0.0)
+    for p, g in zip(prompts, got):
+        toks = list(p)
+        for k in range(n_new):
+            last = plain.forward(cfg, weights, toks)[-1]
+            top = torch.topk(last, 2).values
+            if float(top[0] - top[1]) < 1e-3 * float(last.abs().max()):
+                break                                              # a tie at 32-bit precision: what follows may differ
+            assert g[k] == plain.greedy(last), f"token {k} of a prompt of {len(p)}"
+            toks.append(g[k])
+        assert k >= 5
+
+
+@pytest.mark.gpu
+def test_decode_steps_replay_graphs(models):
+    """Decode steps of one shape are captured and replayed; every replay gives the eager logits."""
+    cfg = CONFIGS["wide"]
+    folder, _ = models("wide", "bfloat16")
+    reqs = requests(cfg["vocab"], [40, 41], 21)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:20], "want": [19]} for r, t in reqs.items()], "end": []}]
+    steps += [{"step": 1 + i, "entries": [{"id": r, "tokens": [t[20 + i]], "want": [0]} for r, t in reqs.items()], "end": []} for i in range(20)]
+    outs = []
+    for graphs in (False, True):
+        eng = engine(folder, "bfloat16", "wide", graphs=graphs)
+        outs.append(H.run_trace_inprocess(eng, copy.deepcopy(steps)))
+        assert (eng.graph_replays > 10) == graphs
+    for k in outs[0]:
+        assert np.array_equal(outs[0][k], outs[1][k]), f"step {k}"
