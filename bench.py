@@ -167,7 +167,8 @@ class KernelTimes:
 
     NAMES = ("embed", "add_rmsnorm", "rope_kvwrite", "router_top1", "moe_plan", "convert", "gemm_generic",
              "attn_generic", "gemm_skinny", "gemm_mfma", "gemm_tiled", "attn_decode", "attn_prefill",
-             "sample_rows", "argmax_rows", "filter_rows")
+             "sample_rows", "argmax_rows", "filter_rows", "latent_prepare", "attn_latent_generic", "attn_latent_mfma",
+             "router_topk", "moe_combine", "gated_rows", "add_into")
 
     def __init__(self):
         import torch
@@ -207,6 +208,129 @@ class KernelTimes:
         rows = sorted(tot.items(), key=lambda kv: -kv[1][0])
         return [{"kernel": k, "ms_per_step": round(t / steps, 4), "calls_per_step": round(n / steps, 1),
                  "share": round(t / whole, 4)} for k, (t, n) in rows]
+
+
+# ---- the Ravenex design beside Llama 4 at equal sizes (``--workload designs``)
+# Sizes that resemble real layers: width, heads, routed experts, experts a token, expert and shared
+# inner widths.  Ravenex: heads of 128 unrotated + 64 rotated elements, values of 128, a latent of
+# 512, a window of 4,096, per-layer token rows of 256, layers in pairs of which the second reads the
+# first one's cache.  Llama 4 at the same width, heads (head size 128, a kv head for every four),
+# experts and layers, its one routed and one shared expert as wide as the Ravenex token's experts
+# together, its rotating layers reading a window of the same length.
+DESIGN_SIZES = {
+    "2k": dict(width=2048, heads=16, experts=16, top=4, expert_ff=1024, shared_ff=2048),
+    "5k": dict(width=5120, heads=40, experts=16, top=2, expert_ff=4096, shared_ff=8192),
+}
+
+
+def design_configs(sz, layers, window, vocab):
+    mix = lambda kv_from: dict({"heads": sz["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+                                "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5},
+                               **({} if kv_from is None else {"kv_from": kv_from}))
+    mlp = {"kind": "moe", "router": {"experts": sz["experts"], "top": sz["top"]}, "expert": {"ff": sz["expert_ff"]},
+           "shared": {"ff": sz["shared_ff"]}}
+    ravenex = {"architecture": "Ravenex", "vocab": vocab, "width": sz["width"], "residual_mult": 0.7, "norm": {"eps": 1e-6},
+               "token_side": {"dim": 256}, "torch_dtype": "bfloat16",
+               "layers": [{"type": "latent_attention", "mixer": mix(None if i % 2 == 0 else i - 1), "mlp": mlp}
+                          for i in range(layers)]}
+    each = (sz["top"] * sz["expert_ff"] + sz["shared_ff"]) // 2
+    llama = dict(SCOUT, num_hidden_layers=layers, hidden_size=sz["width"], num_attention_heads=sz["heads"],
+                 num_key_value_heads=max(1, sz["heads"] // 4), head_dim=128, num_local_experts=sz["experts"],
+                 intermediate_size=each, intermediate_size_mlp=2 * each, vocab_size=vocab, attention_chunk_size=window,
+                 no_rope_layers=None, rope_scaling=None, attention_local_kind="window")
+    return {"ravenex": ravenex, "llama4": llama}
+
+
+def design_comparison(args):
+    """Prefill of one prompt and decode steps of a batch, each design at each size: tokens a second
+    and the time of every kind of kernel in an eager step."""
+    import gc
+
+    import numpy as np
+    import torch
+    from spite_amd.engine.engine import Engine, StepEntry
+    page, V, layers, window = 64, 32768, args.layers or 4, 4096
+    batch, context, T = args.batch, args.context, args.prefill_tokens
+    rng = np.random.RandomState(0)
+    out = {"metric": "prefill and decode tok/s of the Ravenex design beside Llama 4 at equal sizes (random weights)",
+           "value": None, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
+           "higher_is_better": True, "data": "synthetic: random weights, uniform-random token ids, context pages filled with random values",
+           "config": {"layers": layers, "window": window, "global_batch": batch, "seq_len": context, "prefill_tokens": T, "vocab": V},
+           "sizes": {}}
+    for name in [x for x in args.design_sizes.split(",") if x.strip()]:
+        sz = DESIGN_SIZES[name]
+        out["sizes"][name] = {"size": sz}
+        for design, cfg in design_configs(sz, layers, window, V).items():
+            per_req = -(-(context + args.runs * args.steps + args.warmup + 16) // page) * page
+            eng = Engine(cfg, dtype=args.dtype, page_size=page, cache_tokens=max(batch * per_req, T + 2 * page),
+                         max_requests=batch, max_batch_tokens=max(T, batch), random_weights=True, seed=0,
+                         graphs=not args.no_graphs)
+            rec = {"slow_paths": sorted(eng.slow_paths)}
+
+            def prefill_once():
+                s = eng.admit()
+                toks = rng.randint(0, V, size=T).tolist()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                eng.step([StepEntry(s, toks, [T - 1])])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t
+                eng.release(s)
+                return dt
+            prefill_once()
+            pre = statistics.median(prefill_once() for _ in range(max(1, args.runs)))
+            with KernelTimes() as kt:
+                prefill_once()
+                rec["prefill_kernels"] = kt.table(1)
+            rec["prefill"] = {"tokens": T, "ms": round(pre * 1e3, 3), "tok_s": round(T / pre, 1)}
+            slots = [eng.admit() for _ in range(batch)]
+            for s in slots:
+                for at in range(0, context, 2048):
+                    n = min(2048, context - at)
+                    eng.cache.reserve(s, n)
+                    eng.cache.commit(s, n)
+            for g in eng.cache.groups:
+                for half in g.halves():
+                    if half.numel():
+                        half.normal_(0.0, 1.0)
+            toks = rng.randint(0, V, size=batch).tolist()
+
+            def one():
+                nonlocal toks
+                logits = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])
+                toks = torch.argmax(logits, dim=-1).tolist()
+            for _ in range(args.warmup):
+                one()
+            times = []
+            for _ in range(max(1, args.runs)):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(args.steps):
+                    one()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+            dt = statistics.median(times)
+            graphs, eng.use_graphs = eng.use_graphs, False
+            with KernelTimes() as kt:
+                for _ in range(4):
+                    one()
+                rec["decode_kernels"] = kt.table(4)
+            eng.use_graphs = graphs
+            rec["decode"] = {"batch": batch, "context": context, "ms_per_step": round(dt / args.steps * 1e3, 3),
+                             "tok_s": round(batch * args.steps / dt, 1)}
+            log(f"{name} {design}: prefill {T} tokens {pre * 1e3:.2f} ms ({T / pre:.0f} tok/s), decode batch {batch} at {context}: "
+                f"{dt / args.steps * 1e3:.3f} ms/step ({batch * args.steps / dt:.0f} tok/s)")
+            for phase in ("prefill_kernels", "decode_kernels"):
+                for row in rec[phase][:10]:
+                    log(f"    {phase[:-8]} {row['kernel']}: {row['ms_per_step']} ms x{row['calls_per_step']}, {row['share']:.1%}")
+            out["sizes"][name][design] = rec
+            for s in slots:
+                eng.release(s)
+            del eng
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps(out))
+    return 0
 
 
 def sampling_only(V, rows, steps):
@@ -453,7 +577,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--runs", type=int, default=3, help="how many times the K steps are timed")
-    ap.add_argument("--workload", default="decode", choices=["decode", "longctx", "serve"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "longctx", "serve", "designs"],
+                    help="designs: the Ravenex design beside Llama 4 at equal sizes (see DESIGN_SIZES)")
+    ap.add_argument("--design-sizes", default="2k,5k", help="designs: which of DESIGN_SIZES, comma separated")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (memory or time)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
@@ -492,6 +618,8 @@ def main() -> int:
     base = TINY if args.tiny else SCOUT
     if args.phase == "sampling":
         return sampling_only(base["vocab_size"], args.batch, args.steps)
+    if args.workload == "designs":
+        return design_comparison(args)
     if args.workload != "decode":
         print(json.dumps(serving_workload(args, base, Engine, args.runs)))
         return 0

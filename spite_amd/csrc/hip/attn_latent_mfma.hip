@@ -13,6 +13,10 @@
 // Tiles: S^T tile tt (of 2) holds the keys (r/4)*8 + tt*4 + r%4 of the block in its rows r, so the
 // eight scores a lane holds are eight consecutive keys: P^T is the next product's operand without a
 // shuffle.  Scores, maximum, sum and the output are fp32.
+//
+// Few workgroups with many keys (decoded tokens of a few requests over long contexts): the blocks
+// of keys are dealt to `n_splits` workgroups a work item (grid.y), each leaves a record (output not
+// yet divided, maximum, sum) per query row, and a second kernel joins the records.
 #include "common.h"
 
 #define LM_ROWS 128        // query rows per workgroup at most (8 waves of 16)
@@ -23,7 +27,8 @@ __global__ __launch_bounds__(512)
 void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ kv_pages, bf16* __restrict__ out,
                              const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                              const int* __restrict__ block_table, int max_blocks, const int* __restrict__ wg,
-                             int H, int Dk, int R, int ps, int vis, int span, float scale) {
+                             int H, int Dk, int R, int ps, int vis, int span, float scale,
+                             float* __restrict__ part, int n_splits) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int kq = (Dk + 31) >> 5, nv = (R + 15) >> 4;
     const int ks_ld = kq * 32 + 8;                                  // row stride of the staged rows
@@ -71,10 +76,19 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     for (int a = 0; a < NV; ++a) o[a] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int chunks = Dk >> 3;                                     // 16-byte pieces of a row
 
-    for (int blk0 = key_lo & ~31; blk0 <= key_hi; blk0 += 32) {
+    // this workgroup's share of the blocks of keys
+    int blk_first = key_lo >> 5, blk_end = (key_hi >> 5) + 1;
+    if (n_splits > 1) {
+        const int per = (blk_end - blk_first + n_splits - 1) / n_splits;
+        blk_first += (int)blockIdx.y * per;
+        blk_end = blk_first + per < blk_end ? blk_first + per : blk_end;
+    }
+    for (int blk0 = blk_first << 5; blk0 < (blk_end << 5); blk0 += 32) {
         __syncthreads();                                            // the last block's readers are done
+        // consecutive lanes take consecutive keys: the transposed copy's 2-byte stores then fall into
+        // consecutive LDS words instead of one bank
         for (int i = tid; i < 32 * chunks; i += nthreads) {
-            const int key = i / chunks, f = (i - key * chunks) << 3;
+            const int key = i & 31, f = (i >> 5) << 3;
             const int j = blk0 + key;
             bf16x8 v;
 #pragma unroll
@@ -143,6 +157,19 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     }
     if (!row_ok) return;
     // o[a][i] of lane (c, g4) is O[row c][a*16 + g4*4 + i]
+    if (n_splits > 1) {
+        float* rec = part + ((size_t)row * n_splits + blockIdx.y) * (R + 2);
+#pragma unroll
+        for (int a = 0; a < NV; ++a) {
+            const int col = a * 16 + g4 * 4;
+            if (a < nv && col < R) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) rec[col + i] = o[a][i];
+            }
+        }
+        if (g4 == 0) { rec[R] = m_run; rec[R + 1] = l_run; }
+        return;
+    }
     const float inv = 1.0f / fmaxf(l_run, 1e-30f);
     bf16* orow = out + (size_t)row * R;
 #pragma unroll
@@ -157,18 +184,44 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     }
 }
 
+// Joins the records [row][split][R + 2] of a split call: one workgroup a query row.
+__global__ __launch_bounds__(256)
+void attn_latent_join_kernel(const float* __restrict__ part, bf16* __restrict__ out, int R, int n_splits) {
+    const size_t row = blockIdx.x;
+    const float* rec = part + row * n_splits * (R + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, rec[(size_t)s * (R + 2) + R]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float m = rec[(size_t)s * (R + 2) + R];
+        L += (m == -INFINITY ? 0.f : __expf(m - M)) * rec[(size_t)s * (R + 2) + R + 1];
+    }
+    const float inv = 1.0f / fmaxf(L, 1e-30f);
+    for (int c = threadIdx.x; c < R; c += 256) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float m = rec[(size_t)s * (R + 2) + R];
+            if (m != -INFINITY) acc += __expf(m - M) * rec[(size_t)s * (R + 2) + c];
+        }
+        out[row * R + c] = (bf16)(acc * inv);
+    }
+}
+
 // `wg`: int32 pairs (first query row, rows <= 128) on the device, `n_wg` of them, each within one
 // request's rows of the step; `max_rows`: the most rows of any pair (it sizes the workgroups).
+// `n_splits` > 1: the keys of every pair are dealt to that many workgroups; `part` (fp32,
+// rows * n_splits * (R + 2) floats, rows = T * H) holds their records.
 extern "C" int spite_attn_latent_mfma(const void* q, const void* kv_pages, void* out, const int* positions,
                                       const int* seq_of_token, const int* block_table, int max_blocks, const int* wg,
                                       int n_wg, int max_rows, int H, int Dk, int R, int page_size, int vis, int span,
-                                      float scale, hipStream_t st) {
+                                      float scale, float* part, int n_splits, int n_rows, hipStream_t st) {
     SP_REQUIRE(H > 0 && n_wg >= 0 && max_rows >= 0 && max_rows <= LM_ROWS, "latent attention: %d rows a workgroup, at most %d", max_rows, LM_ROWS);
     SP_REQUIRE(Dk > 0 && Dk % 8 == 0 && R > 0 && R % 8 == 0 && R <= Dk && Dk <= 576 && R <= 512,
                "latent attention (MFMA): rows of %d with a latent of %d: multiples of 8, at most 576 and 512", Dk, R);
     SP_REQUIRE(page_size > 0 && max_blocks > 0, "latent attention: bad page size %d or table width %d", page_size, max_blocks);
     SP_REQUIRE(vis >= 0 && vis < SP_VIS_COUNT && (!sp_vis_has_span(vis) || span > 0), "latent attention: chunk or window of %d", span);
     SP_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kv_pages & 15) == 0 && ((uintptr_t)out & 7) == 0, "latent attention: operands must be 16-byte aligned");
+    SP_REQUIRE(n_splits >= 1 && n_splits <= 1024 && (n_splits == 1 || part), "latent attention: %d splits", n_splits);
     if (n_wg == 0 || max_rows == 0) return 0;
     const int kq = (Dk + 31) / 32, nv = (R + 15) / 16;
     const int nw = (max_rows + 15) / 16;
@@ -178,12 +231,16 @@ extern "C" int spite_attn_latent_mfma(const void* q, const void* kv_pages, void*
         static bool allowed = false; \
         if (sh > 48 * 1024 && !allowed) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
             if (e != hipSuccess) return sp_fail("latent attention: %zu bytes of LDS refused: %s", sh, hipGetErrorString(e)); allowed = true; } \
-        kern<<<n_wg, nw * 64, sh, st>>>((const bf16*)q, (const bf16*)kv_pages, (bf16*)out, positions, seq_of_token, \
-                                        block_table, max_blocks, wg, H, Dk, R, page_size, vis, span, scale); } while (0)
+        kern<<<dim3(n_wg, n_splits), nw * 64, sh, st>>>((const bf16*)q, (const bf16*)kv_pages, (bf16*)out, positions, seq_of_token, \
+                                        block_table, max_blocks, wg, H, Dk, R, page_size, vis, span, scale, part, n_splits); } while (0)
     if (kq <= 6 && nv <= 8) SP_LM(6, 8);
     else if (kq <= 10 && nv <= 16) SP_LM(10, 16);
     else SP_LM(18, 32);
 #undef SP_LM
     SP_LAUNCH_CHECK("attn_latent_mfma");
+    if (n_splits > 1) {
+        attn_latent_join_kernel<<<n_rows, 256, 0, st>>>(part, (bf16*)out, R, n_splits);
+        SP_LAUNCH_CHECK("attn_latent_join");
+    }
     return 0;
 }

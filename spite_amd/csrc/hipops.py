@@ -59,7 +59,7 @@ def lib():
             "spite_mfma_loop": [P, I, I, F, P],
             "spite_latent_prepare": [P, I, P, I, P, P, I, P, P, P, P, F, I, I, I, I, I, I, I, P, P, P],
             "spite_attn_latent_generic": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
-            "spite_attn_latent_mfma": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, F, P],
+            "spite_attn_latent_mfma": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, F, P, I, I, P],
             "spite_router_topk": [P, P, P, P, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
@@ -711,9 +711,24 @@ def latent_workgroups(counts, cu_seqlens, H):
     return np.asarray(out, dtype=np.int32), (len(out) // 2, most)
 
 
-def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg, n_wg, max_rows, T, H, Dk, R, vis, span, scale):
+def latent_splits(n_wg: int, longest: int) -> int:
+    """Into how many workgroups the keys of every work item are best dealt, for ``n_wg`` items whose
+    queries read at most ``longest`` keys: about two workgroups a compute unit, each with at least
+    two blocks of 32 keys."""
+    if n_wg <= 0:
+        return 1
+    return max(1, min(-(-2 * cu_count() // n_wg), -(-longest // 64), 256))
+
+
+def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg, n_wg, max_rows, T, H, Dk, R, vis, span, scale,
+                     n_splits=1, scratch=None):
     """As ``attn_latent_generic`` on the matrix units (bfloat16; see ``attn_latent_mfma_ok``).  ``wg``:
-    the work list of ``latent_workgroups`` on the device."""
+    the work list of ``latent_workgroups`` on the device.  ``n_splits`` > 1 (``latent_splits``) deals
+    every item's keys to that many workgroups; ``scratch`` (fp32, T*H*n_splits*(R+2) elements) then
+    holds their records."""
+    n_splits = int(n_splits)
+    if n_splits > 1 and (scratch is None or scratch.dtype != torch.float32 or scratch.numel() < T * H * n_splits * (R + 2)):
+        raise KernelError(f"latent attention (MFMA): {n_splits} splits need {T * H * n_splits * (R + 2)} floats of scratch")
     _latent_checks(q, kv_pages, out, positions, seq_of_token, block_table, T, H, Dk, R, "latent attention (MFMA)")
     if q.dtype != torch.bfloat16:
         raise KernelError(f"latent attention (MFMA): bfloat16 only, got {q.dtype}")
@@ -724,4 +739,5 @@ def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg,
         _ptr(q, "q", dt), _ptr(kv_pages, "kv_pages", dt), _ptr(out, "out", dt), _ptr(positions, "positions", torch.int32),
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], _ptr(wg, "wg", torch.int32), int(n_wg), int(max_rows), H, Dk, R, kv_pages.shape[2],
-        VIS[vis], int(span or 0), float(scale), _stream()), "latent attention (MFMA)")
+        VIS[vis], int(span or 0), float(scale), _ptr(scratch, "scratch", torch.float32) if n_splits > 1 else None,
+        n_splits, T * H, _stream()), "latent attention (MFMA)")

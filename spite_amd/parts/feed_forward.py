@@ -234,8 +234,15 @@ class MoeTopKSigmoid(FeedForward):
             hipops.gemm_generic(x32, self.w_router, logits, T, E, d)
         n = T * k
         expert, weight = ws.take((n,), torch.int32), ws.take((n,), torch.float32)
-        hipops.router_topk(logits, self.bias, expert, weight, k, renorm=self.renormalize)
         trace = ctx.extras.get("trace")
+        bias = self.bias
+        if trace is not None and trace.get("take_experts"):
+            # a testing aid: the experts are given ([T, top_k] per call, in the order of the calls), each
+            # with the weight that its own logit gives; every other logit is taken out of the choice
+            take = trace["take_experts"].pop(0).to(device=x.device, dtype=torch.int64).view(T, k)
+            logits = torch.full_like(logits, float("-inf")).scatter_(1, take, logits.gather(1, take))
+            bias = None
+        hipops.router_topk(logits, bias, expert, weight, k, renorm=self.renormalize)
         if trace is not None:                         # a testing aid: which experts each token took, [T, top_k]
             trace.setdefault("moe_experts", []).append(expert.view(T, k).clone())
         src, dst, unused = ws.take((n,), torch.int32), ws.take((n,), torch.int32), ws.take((n,), torch.float32)

@@ -130,8 +130,16 @@ class LatentAttention(Mixer):
         o_lat = ws.take((T * H, R), x.dtype)
         if self.mfma:
             wg, (n_wg, most) = ctx.derived[self._wg]
+            # the most keys that a query of the step may read, bounded by the block table's width (the same
+            # for every step of one shape) and by the layer's reach
+            longest = cache.block_table.shape[1] * cache.page_size
+            if self.visibility != "full":
+                longest = min(longest, self.span + ctx.max_count + 31)
+            n_splits = hipops.latent_splits(n_wg, longest)
+            scratch = ws.take((T * H * n_splits * (R + 2),), torch.float32) if n_splits > 1 else None
             hipops.attn_latent_mfma(qa, cache.k_pages, o_lat, ctx.positions, ctx.seq_of_token, cache.block_table,
-                                    wg, n_wg, most, T, H, Dk, R, self.visibility, self.span, self.scale)
+                                    wg, n_wg, most, T, H, Dk, R, self.visibility, self.span, self.scale,
+                                    n_splits=n_splits, scratch=scratch)
         else:
             hipops.attn_latent_generic(qa, cache.k_pages, o_lat, ctx.positions, ctx.seq_of_token, cache.block_table,
                                        T, H, Dk, R, self.visibility, self.span, self.scale)

@@ -279,13 +279,15 @@ def test_latent_attention_matrix_kernel(Hh, Dk, R, ps, vis, span):
     c = _attention_case(Hh, Dk, R, ps, [1, 37, 1, 70, 2], [199, 0, 0, 45, 63], vis, span, "bfloat16", Dk + Hh)
     wg, (n_wg, most) = hipops.latent_workgroups(c["counts"], c["cu"], Hh)
     assert most <= hipops.LATENT_WG_ROWS and int(wg[1::2].sum()) == c["T"] * Hh
-    out = torch.full((c["T"] * Hh, R), float("nan"), device="cuda:0", dtype=torch.bfloat16)
-    hipops.attn_latent_mfma(c["q"], c["pages"], out, c["positions"], c["seq"], c["table"], torch.from_numpy(wg).cuda(), n_wg, most,
-                            c["T"], Hh, Dk, R, vis, span, c["scale"])
+    tol = 0.02 * float(c["want"].abs().max())
+    for n_splits in (1, 3, 8):                     # the keys of every work item in one workgroup, or dealt to several
+        out = torch.full((c["T"] * Hh, R), float("nan"), device="cuda:0", dtype=torch.bfloat16)
+        scratch = torch.full((c["T"] * Hh * n_splits * (R + 2),), float("nan"), device="cuda:0") if n_splits > 1 else None
+        hipops.attn_latent_mfma(c["q"], c["pages"], out, c["positions"], c["seq"], c["table"], torch.from_numpy(wg).cuda(), n_wg, most,
+                                c["T"], Hh, Dk, R, vis, span, c["scale"], n_splits=n_splits, scratch=scratch)
+        assert float((out.cpu().double() - c["want"]).abs().max()) < tol, f"{n_splits} splits"
     ref = torch.empty_like(out)
     hipops.attn_latent_generic(c["q"], c["pages"], ref, c["positions"], c["seq"], c["table"], c["T"], Hh, Dk, R, vis, span, c["scale"])
-    tol = 0.02 * float(c["want"].abs().max())
-    assert float((out.cpu().double() - c["want"]).abs().max()) < tol
     assert float((ref.cpu().double() - c["want"]).abs().max()) < tol
 
 
@@ -351,7 +353,18 @@ def test_bfloat16_against_plain_and_itself(models, name):
     err, where = H.max_diff(rows, ref)
     assert err <= 0.05 * scale, f"{err} at {where} (scale {scale})"
     for steps in (H.schedule_tail_one_by_one(reqs, tail=28), H.schedule_portions(reqs), H.schedule_mixed(reqs, seed=4, max_live=4)):
-        got = H.collect(steps, H.run_trace_inprocess(eng, steps), cfg["vocab"])
+        # the experts of the whole prompts are taken again: a choice between two scores that are tied at
+        # this precision may fall either way from one schedule to the next
+        fed, take = {}, {}
+        for rec in steps:
+            per_layer = [[] for _ in moe]
+            for e in rec["entries"]:
+                at, n = fed.get(e["id"], 0), len(e["tokens"])
+                for k, L in enumerate(moe):
+                    per_layer[k].append(experts[e["id"]][L][at:at + n].numpy())
+                fed[e["id"]] = at + n
+            take[rec["step"]] = [np.concatenate(x) for x in per_layer]
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps, take=take), cfg["vocab"])
         err, where = H.max_diff(got, rows)
         assert err <= 0.05 * scale, f"{err} at {where} (scale {scale})"
 
