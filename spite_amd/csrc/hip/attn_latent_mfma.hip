@@ -83,30 +83,49 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         blk_first += (int)blockIdx.y * per;
         blk_end = blk_first + per < blk_end ? blk_first + per : blk_end;
     }
+    // Staging: a thread keeps one key of the block (consecutive lanes take consecutive keys, so the
+    // transposed copy's 2-byte stores fall into consecutive LDS words instead of one bank) and walks
+    // that key's 16-byte pieces.  Where the key's row lies is looked up one block ahead, so the table
+    // entry's way from memory is hidden behind the block before.
+    const int key = tid & 31, piece0 = tid >> 5, piece_step = nthreads >> 5;
+    // LDS row of a key: the 16 rows of S^T tile tt lie together, tile row (key/8)*4 + key%4
+    bf16* ks_row = Ks + ((((key >> 2) & 1) << 4) + ((key >> 3) << 2) + (key & 3)) * ks_ld;
+    auto row_of = [&](int blk0) -> long long {       // first element of the key's cache row; -1: page given back; -2: not read
+        const int j = blk0 + key;
+        if (j < key_lo || j > key_hi) return -2;
+        const int page = bt[j / ps];
+        return page >= 0 ? ((long long)page * ps + j % ps) * Dk : -1;
+    };
+    long long row_cur = blk_first < blk_end ? row_of(blk_first << 5) : -2;
     for (int blk0 = blk_first << 5; blk0 < (blk_end << 5); blk0 += 32) {
+        const long long row_next = blk0 + 32 < (blk_end << 5) ? row_of(blk0 + 32) : -2;
         __syncthreads();                                            // the last block's readers are done
-        // consecutive lanes take consecutive keys: the transposed copy's 2-byte stores then fall into
-        // consecutive LDS words instead of one bank
-        for (int i = tid; i < 32 * chunks; i += nthreads) {
-            const int key = i & 31, f = (i >> 5) << 3;
-            const int j = blk0 + key;
-            bf16x8 v;
+        const bf16* src = kv_pages + (row_cur >= 0 ? row_cur : 0);
+        for (int pc = piece0; pc < chunks; pc += 2 * piece_step) {  // two loads in flight before their stores
+            const int f0 = pc << 3, f1 = (pc + piece_step) << 3;
+            bf16x8 v0, v1;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (bf16)0.f;
-            int gone = 0;
-            if (j >= key_lo && j <= key_hi) {
-                const int page = bt[j / ps];
-                if (page >= 0) v = *(const bf16x8*)(kv_pages + ((size_t)page * ps + j % ps) * Dk + f);
-                else gone = 1;
+            for (int e = 0; e < 8; ++e) { v0[e] = (bf16)0.f; v1[e] = (bf16)0.f; }
+            const bool two = pc + piece_step < chunks;
+            if (row_cur >= 0) {
+                v0 = *(const bf16x8*)(src + f0);
+                if (two) v1 = *(const bf16x8*)(src + f1);
             }
-            // LDS row of a key: the 16 rows of S^T tile tt lie together, tile row (key/8)*4 + key%4
-            *(bf16x8*)(Ks + ((((key >> 2) & 1) << 4) + ((key >> 3) << 2) + (key & 3)) * ks_ld + f) = v;
-            if (f < R) {
+            *(bf16x8*)(ks_row + f0) = v0;
+            if (f0 < R) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) Vt[(f + e) * LM_VT_LD + key] = v[e];
+                for (int e = 0; e < 8; ++e) Vt[(f0 + e) * LM_VT_LD + key] = v0[e];
             }
-            if (f == 0) kflag[key] = gone;
+            if (two) {
+                *(bf16x8*)(ks_row + f1) = v1;
+                if (f1 < R) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) Vt[(f1 + e) * LM_VT_LD + key] = v1[e];
+                }
+            }
         }
+        if (tid < 32) kflag[key] = row_cur == -1;
+        row_cur = row_next;
         __syncthreads();
         if (blk0 + 31 < wave_lo || blk0 > wave_hi) continue;        // nothing here for this wave's rows
 
@@ -187,21 +206,41 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
 // Joins the records [row][split][R + 2] of a split call: one workgroup a query row.
 __global__ __launch_bounds__(256)
 void attn_latent_join_kernel(const float* __restrict__ part, bf16* __restrict__ out, int R, int n_splits) {
+    __shared__ float wsh[1024];          // weight of every split: exp(m_s - M) / L
+    __shared__ float red[8];
     const size_t row = blockIdx.x;
     const float* rec = part + row * n_splits * (R + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, rec[(size_t)s * (R + 2) + R]);
-    float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float m = rec[(size_t)s * (R + 2) + R];
-        L += (m == -INFINITY ? 0.f : __expf(m - M)) * rec[(size_t)s * (R + 2) + R + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the first 1024 splits' maxima and sums, four a thread
+    float ms[4], ls[4], M = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int s = tid + u * 256;
+        ms[u] = s < n_splits ? rec[(size_t)s * (R + 2) + R] : -INFINITY;
+        ls[u] = s < n_splits ? rec[(size_t)s * (R + 2) + R + 1] : 0.f;
+        M = fmaxf(M, ms[u]);
     }
-    const float inv = 1.0f / fmaxf(L, 1e-30f);
-    for (int c = threadIdx.x; c < R; c += 256) {
+    M = wave_max(M);
+    if (lane == 0) red[wave] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float L = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int s = tid + u * 256;
+        const float w = ms[u] == -INFINITY ? 0.f : __expf(ms[u] - M);
+        if (s < n_splits) wsh[s] = w;
+        L += w * ls[u];
+    }
+    L = wave_sum(L);
+    if (lane == 0) red[4 + wave] = L;
+    __syncthreads();
+    const float inv = 1.0f / fmaxf(red[4] + red[5] + red[6] + red[7], 1e-30f);
+    for (int c = tid; c < R; c += 256) {
         float acc = 0.f;
         for (int s = 0; s < n_splits; ++s) {
-            const float m = rec[(size_t)s * (R + 2) + R];
-            if (m != -INFINITY) acc += __expf(m - M) * rec[(size_t)s * (R + 2) + c];
+            const float w = wsh[s];
+            if (w != 0.f) acc += w * rec[(size_t)s * (R + 2) + c];
         }
         out[row * R + c] = (bf16)(acc * inv);
     }
@@ -224,7 +263,11 @@ extern "C" int spite_attn_latent_mfma(const void* q, const void* kv_pages, void*
     SP_REQUIRE(n_splits >= 1 && n_splits <= 1024 && (n_splits == 1 || part), "latent attention: %d splits", n_splits);
     if (n_wg == 0 || max_rows == 0) return 0;
     const int kq = (Dk + 31) / 32, nv = (R + 15) / 16;
-    const int nw = (max_rows + 15) / 16;
+    // a wave for every 16 query rows, and enough waves that staging a block of 32 keys takes a thread
+    // no more than about four 16-byte pieces (waves without rows only stage)
+    int nw = (max_rows + 15) / 16;
+    const int stage_waves = (32 * (Dk / 8) + 255) / 256;
+    if (nw < stage_waves) nw = stage_waves < 8 ? stage_waves : 8;
     const size_t sh = ((size_t)32 * (kq * 32 + 8) + (size_t)nv * 16 * LM_VT_LD) * sizeof(bf16) + 32 * sizeof(int);
 #define SP_LM(KQV, NVV) do { \
         auto kern = attn_latent_mfma_kernel<KQV, NVV>; \

@@ -713,11 +713,11 @@ def latent_workgroups(counts, cu_seqlens, H):
 
 def latent_splits(n_wg: int, longest: int) -> int:
     """Into how many workgroups the keys of every work item are best dealt, for ``n_wg`` items whose
-    queries read at most ``longest`` keys: about two workgroups a compute unit, each with at least
-    two blocks of 32 keys."""
+    queries read at most ``longest`` keys: about one workgroup a compute unit, each with at least eight
+    blocks of 32 keys (a workgroup's record is as large as what it reads of two or three such blocks)."""
     if n_wg <= 0:
         return 1
-    return max(1, min(-(-2 * cu_count() // n_wg), -(-longest // 64), 256))
+    return max(1, min(-(-cu_count() // n_wg), -(-longest // 256), 256))
 
 
 def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg, n_wg, max_rows, T, H, Dk, R, vis, span, scale,
