@@ -96,33 +96,29 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         const int page = bt[j / ps];
         return page >= 0 ? ((long long)page * ps + j % ps) * Dk : -1;
     };
+    auto put = [&](int f, const bf16x8& v) {
+        *(bf16x8*)(ks_row + f) = v;
+        if (f < R) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) Vt[(f + e) * LM_VT_LD + key] = v[e];
+        }
+    };
     long long row_cur = blk_first < blk_end ? row_of(blk_first << 5) : -2;
     for (int blk0 = blk_first << 5; blk0 < (blk_end << 5); blk0 += 32) {
         const long long row_next = blk0 + 32 < (blk_end << 5) ? row_of(blk0 + 32) : -2;
         __syncthreads();                                            // the last block's readers are done
         const bf16* src = kv_pages + (row_cur >= 0 ? row_cur : 0);
         for (int pc = piece0; pc < chunks; pc += 2 * piece_step) {  // two loads in flight before their stores
-            const int f0 = pc << 3, f1 = (pc + piece_step) << 3;
             bf16x8 v0, v1;
 #pragma unroll
             for (int e = 0; e < 8; ++e) { v0[e] = (bf16)0.f; v1[e] = (bf16)0.f; }
             const bool two = pc + piece_step < chunks;
             if (row_cur >= 0) {
-                v0 = *(const bf16x8*)(src + f0);
-                if (two) v1 = *(const bf16x8*)(src + f1);
+                v0 = *(const bf16x8*)(src + (pc << 3));
+                if (two) v1 = *(const bf16x8*)(src + ((pc + piece_step) << 3));
             }
-            *(bf16x8*)(ks_row + f0) = v0;
-            if (f0 < R) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) Vt[(f0 + e) * LM_VT_LD + key] = v0[e];
-            }
-            if (two) {
-                *(bf16x8*)(ks_row + f1) = v1;
-                if (f1 < R) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) Vt[(f1 + e) * LM_VT_LD + key] = v1[e];
-                }
-            }
+            put(pc << 3, v0);
+            if (two) put((pc + piece_step) << 3, v1);
         }
         if (tid < 32) kflag[key] = row_cur == -1;
         row_cur = row_next;
