@@ -459,3 +459,115 @@ def test_decode_steps_replay_graphs(models):
         assert (eng.graph_replays > 10) == graphs
     for k in outs[0]:
         assert np.array_equal(outs[0][k], outs[1][k]), f"step {k}"
+
+
+def random_config(seed, aligned=False):
+    """A configuration drawn from a seed: layer count and order, heads, sizes, windows, bases, experts and
+    constants all vary; now and then a value is 1 (one head, a window of one key, one expert, all experts
+    taken) or sizes are odd.  ``aligned``: sizes in multiples of 8, 16 and 64, which the bfloat16 runs
+    take on the matrix units in one kernel or another."""
+    rng = np.random.RandomState(seed)
+    pick = lambda *xs: xs[rng.randint(len(xs))]
+    if aligned:
+        width = int(pick(64, 128, 192, 256))
+        layers, owners = [], []
+        for i in range(int(pick(2, 3, 4))):
+            if owners and rng.rand() < 0.4:
+                j = int(pick(*owners))
+                src = layers[j]["mixer"]
+                rank, rot, base, kv_from = src["kv_rank"], src["rot_dim"], src["rot"]["base"], j
+            else:
+                rank, rot, base, kv_from = int(pick(16, 32, 64, 96, 128)), int(pick(8, 16, 32)), float(pick(1000.0, 10000.0)), None
+                owners.append(i)
+            mix = _mixer(int(pick(2, 4, 6, 17)), int(pick(8, 16, 32, 64)), rot, int(pick(8, 16, 32, 48)), rank,
+                         pick(None, 24, 72, 100), kv_from=kv_from, base=base)
+            kind = pick("dense", "moe", "moe")
+            mlp = {"kind": "dense", "ff": int(pick(32, 64, 128, 200))} if kind == "dense" else \
+                _moe(int(pick(4, 8, 12)), int(pick(1, 2, 3)), int(pick(16, 32, 64)), pick(None, 48, 64))
+            layers.append(_layer(mix, mlp))
+        return {"architecture": "Ravenex", "vocab": int(pick(256, 640)), "width": width, "residual_mult": float(pick(0.7, 1.0)),
+                "norm": {"eps": 1e-6}, "token_side": pick(None, {"dim": 8}, {"dim": 24}), "layers": layers}
+    width = int(pick(24, 37, 48, 64, 96))
+    layers, owners = [], []
+    for i in range(int(pick(1, 2, 3, 5, 6))):
+        if owners and rng.rand() < 0.45:
+            j = int(pick(*owners))
+            src = layers[j]["mixer"]
+            rank, rot, base = src["kv_rank"], src["rot_dim"], src["rot"]["base"]
+            kv_from = j
+        else:
+            rank, rot, base, kv_from = int(pick(4, 8, 12, 24, 32)), int(pick(2, 4, 8, 16)), float(pick(100.0, 10000.0, 5e5)), None
+            owners.append(i)
+        mix = _mixer(int(pick(1, 2, 3, 5, 8)), int(pick(2, 6, 8, 16, 24)), rot, int(pick(1, 4, 8, 10, 16)), rank,
+                     pick(None, 1, 2, 7, 16, 33, 64), kv_from=kv_from, base=base, scale=float(pick(0.1, 0.25, 0.5)))
+        kind = pick("dense", "moe", "moe", None)
+        if kind == "dense":
+            mlp = {"kind": "dense", "ff": int(pick(8, 20, 32, 64))}
+        elif kind == "moe":
+            E = int(pick(1, 2, 4, 7, 9))
+            mlp = _moe(E, int(pick(*range(1, E + 1))), int(pick(4, 8, 16, 24)), pick(None, 8, 12, 32))
+        else:
+            mlp = None
+        layers.append(_layer(mix, mlp))
+    return {"architecture": "Ravenex", "vocab": int(pick(50, 128, 257)), "width": width, "residual_mult": float(pick(0.5, 1.0, 1.7)),
+            "norm": {"eps": float(pick(1e-6, 1e-5, 1e-3))}, "token_side": pick(None, {"dim": 1}, {"dim": 5}, {"dim": 8}), "layers": layers}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(12)) + list(range(100, 110)))
+def test_random_configurations(tmp_path, seed):
+    """Whatever the configuration says: true 32-bit against the plain implementation, whole prompts and a
+    mixed schedule through small pages; then bfloat16 against itself across schedules (the whole prompts'
+    experts taken again) and, loosely, against the plain implementation."""
+    cfg = random_config(seed, aligned=seed >= 100)
+    page = int(np.random.RandomState(seed + 100).choice([4, 16, 32, 64]))
+    weights = make_model(tmp_path / "f32", cfg, seed=seed, dtype="float32", qk_gain=2.0)
+    reqs = requests(cfg["vocab"], [41, 1, 70, 2, 19], seed)
+    ref = plain_rows(cfg, weights, reqs)
+    from spite_amd import Engine
+    eng = Engine(str(tmp_path / "f32"), dtype="float32", page_size=page, cache_tokens=4 * (70 + page), max_requests=4, device="cuda:0")
+    poison(eng)
+    for steps in (H.schedule_whole(reqs), H.schedule_mixed(reqs, seed=seed, max_live=4)):
+        got = H.collect(steps, H.run_trace_inprocess(eng, steps), cfg["vocab"])
+        err, where = H.max_diff(got, ref)
+        assert err <= 3e-4 * scale_of(ref), f"{err} at {where} (scale {scale_of(ref)}): {cfg}"
+    del eng
+    weights = make_model(tmp_path / "bf16", cfg, seed=seed, dtype="bfloat16", qk_gain=1.5, router_gain=4.0, std=0.05)
+    eng = Engine(str(tmp_path / "bf16"), dtype="bfloat16", page_size=page, cache_tokens=4 * (70 + page), max_requests=4, device="cuda:0")
+    poison(eng)
+    whole, routing = H.schedule_whole(reqs), {}
+    rows = H.collect(whole, H.run_trace_inprocess(eng, whole, routing), cfg["vocab"])
+    moe = [i for i, L in enumerate(cfg["layers"]) if L["mlp"] and L["mlp"]["kind"] == "moe"]
+    experts = {rec["entries"][0]["id"]: {L: torch.from_numpy(routing[rec["step"]][k]).long() for k, L in enumerate(moe)} for rec in whole}
+    ref = plain_rows(cfg, weights, reqs, experts)
+    scale = scale_of(ref)
+    err, where = H.max_diff(rows, ref)
+    assert err <= 0.08 * scale, f"{err} at {where} (scale {scale}): {cfg}"
+    steps = H.schedule_mixed(reqs, seed=seed + 1, max_live=4)
+    fed, take = {}, {}
+    for rec in steps:
+        per_layer = [[] for _ in moe]
+        for e in rec["entries"]:
+            at, n = fed.get(e["id"], 0), len(e["tokens"])
+            for k, L in enumerate(moe):
+                per_layer[k].append(experts[e["id"]][L][at:at + n].numpy())
+            fed[e["id"]] = at + n
+        take[rec["step"]] = [np.concatenate(x) for x in per_layer]
+    got = H.collect(steps, H.run_trace_inprocess(eng, steps, take=take), cfg["vocab"])
+    err, where = H.max_diff(got, rows)
+    assert err <= 0.08 * scale, f"{err} at {where} (scale {scale}): {cfg}"
+
+
+@pytest.mark.gpu
+def test_replay_program(models):
+    """The replay program on a model folder, as a child process: a mixed schedule in true 32-bit gives the
+    plain implementation's logits."""
+    cfg = CONFIGS["small"]
+    folder, weights = models("small", "float32")
+    reqs = requests(cfg["vocab"], [30, 1, 47, 12, 22], 77)
+    steps = H.schedule_mixed(reqs, seed=9, max_live=4)
+    out = H.run_trace_program(str(folder), "float32", steps, max_tokens=4 * 64, extra=["--page-size", "16", "--max-requests", "4"])
+    got = H.collect(steps, out, cfg["vocab"])
+    ref = plain_rows(cfg, weights, reqs)
+    err, where = H.max_diff(got, ref)
+    assert err <= 2e-4 * scale_of(ref), f"{err} at {where}"
