@@ -20,6 +20,8 @@
 #include "common.h"
 
 #define LM_ROWS 128        // query rows per workgroup at most (8 waves of 16)
+#define LM_PRE 12          // 16-byte pieces of a key's row that a staging thread keeps in registers, per block in flight
+#define LM_KROW_BLOCKS 128 // blocks of keys whose cache rows the staging waves look up ahead of their loop
 #define LM_VT_LD 40        // row stride of the transposed values in LDS (32 keys + 8: no bank conflicts, 16-byte rows)
 
 template <int KQ, int NV>   // Dk <= 32*KQ, R <= 16*NV
@@ -35,13 +37,88 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     bf16* Ks = (bf16*)lds_raw;                                      // [32][ks_ld]
     bf16* Vt = Ks + 32 * ks_ld;                                     // [nv*16][LM_VT_LD]
     int* kflag = (int*)(Vt + nv * 16 * LM_VT_LD);                   // [32] 1: the key's page was given back
+    int* krow = kflag + 32;                                         // [LM_KROW_BLOCKS * 32] cache rows of the share's keys (staging waves)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
-    const int c = lane & 15, g4 = lane >> 4;
     const int row0 = wg[2 * blockIdx.x], nrows = wg[2 * blockIdx.x + 1];
     const int t_first = row0 / H, t_last = (row0 + nrows - 1) / H;
     const int* bt = block_table + (size_t)seq_of_token[t_first] * max_blocks;
     const int key_lo = sp_first_visible(positions[t_first], vis, span), key_hi = positions[t_last];
 
+    // the staged rows' elements past Dk are zero for good
+    for (int i = tid; i < 32 * (ks_ld - Dk); i += nthreads) {
+        const int key = i / (ks_ld - Dk), f = Dk + i % (ks_ld - Dk);
+        Ks[key * ks_ld + f] = (bf16)0.f;
+    }
+    for (int i = tid; i < (nv * 16 - R) * LM_VT_LD; i += nthreads) Vt[R * LM_VT_LD + i] = (bf16)0.f;
+
+    const int chunks = Dk >> 3;                                     // 16-byte pieces of a row
+
+    // this workgroup's share of the blocks of keys
+    int blk_first = key_lo >> 5, blk_end = (key_hi >> 5) + 1;
+    if (n_splits > 1) {
+        const int per = (blk_end - blk_first + n_splits - 1) / n_splits;
+        blk_first += (int)blockIdx.y * per;
+        blk_end = blk_first + per < blk_end ? blk_first + per : blk_end;
+    }
+    // Waves beyond the ones that hold query rows do all the staging when they can keep a block's
+    // pieces in registers (2 threads a key and wave, PRE pieces a thread) and the share's cache rows
+    // fit their table: they fetch the next two blocks while the others compute on this one.  Their loop
+    // holds no load but the rows' own, so nothing makes them wait for the youngest load; the table
+    // entries of the whole share are looked up before it.
+    constexpr int PRE = KQ <= 6 ? 4 : (KQ <= 10 ? 8 : LM_PRE);      // smaller rows leave the other instantiations their registers
+    const int n_cw = (nrows + 15) >> 4, n_lw = (nthreads >> 6) - n_cw, n_blk = blk_end - blk_first;
+    const bool roles = n_lw * 2 * PRE >= chunks && n_blk <= LM_KROW_BLOCKS && n_blk > 0;
+    if (roles && wave >= n_cw) {
+        const int lt = tid - n_cw * 64, key = lt & 31, piece0 = lt >> 5, piece_step = n_lw * 2;
+        bf16* ks_row = Ks + ((((key >> 2) & 1) << 4) + ((key >> 3) << 2) + (key & 3)) * ks_ld;
+        for (int i = lt; i < n_blk * 32; i += n_lw * 64) {
+            const int j = (blk_first << 5) + i;
+            int r = -2;
+            if (j >= key_lo && j <= key_hi) { const int page = bt[j / ps]; r = page >= 0 ? page * ps + j % ps : -1; }
+            krow[i] = r;
+        }
+        __syncthreads();                                            // (the rows' waves meet it before their loop)
+        bf16x8 preA[PRE], preB[PRE];
+        auto fetch = [&](bf16x8* pre, int r) {
+#pragma unroll
+            for (int u = 0; u < PRE; ++u) {
+                const int pc = piece0 + u * piece_step;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pre[u][e] = (bf16)0.f;
+                if (r >= 0 && pc < chunks) pre[u] = *(const bf16x8*)(kv_pages + (size_t)r * Dk + (pc << 3));
+            }
+        };
+        auto stage = [&](const bf16x8* pre, int r) {
+            __syncthreads();                                        // the last block's readers are done
+#pragma unroll
+            for (int u = 0; u < PRE; ++u) {
+                const int pc = piece0 + u * piece_step, f = pc << 3;
+                if (pc < chunks) {
+                    *(bf16x8*)(ks_row + f) = pre[u];
+                    if (f < R) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) Vt[(f + e) * LM_VT_LD + key] = pre[u][e];
+                    }
+                }
+            }
+            if (lt < 32) kflag[key] = r == -1;
+            __syncthreads();
+        };
+        int rA = krow[key], rB = n_blk > 1 ? krow[32 + key] : -2;
+        fetch(preA, rA);
+        if (n_blk > 1) fetch(preB, rB);
+        for (int b = 0; b < n_blk; b += 2) {
+            stage(preA, rA);
+            if (b + 2 < n_blk) { rA = krow[(b + 2) * 32 + key]; fetch(preA, rA); }   // on its way while the others compute
+            if (b + 1 < n_blk) {
+                stage(preB, rB);
+                if (b + 3 < n_blk) { rB = krow[(b + 3) * 32 + key]; fetch(preB, rB); }
+            }
+        }
+        return;
+    }
+
+    const int c = lane & 15, g4 = lane >> 4;
     // this lane's query row: a column of every tile
     const int my = wave * 16 + c;
     const bool row_ok = my < nrows;
@@ -63,26 +140,10 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         for (int e = 0; e < 8; ++e) z[e] = (bf16)0.f;
         qf[k] = (k < kq && f < Dk) ? *(const bf16x8*)(q + (size_t)row * Dk + f) : z;
     }
-    // the staged rows' elements past Dk are zero for good
-    for (int i = tid; i < 32 * (ks_ld - Dk); i += nthreads) {
-        const int key = i / (ks_ld - Dk), f = Dk + i % (ks_ld - Dk);
-        Ks[key * ks_ld + f] = (bf16)0.f;
-    }
-    for (int i = tid; i < (nv * 16 - R) * LM_VT_LD; i += nthreads) Vt[R * LM_VT_LD + i] = (bf16)0.f;
-
     float m_run = -INFINITY, l_run = 0.f;
     f32x4 o[NV];
 #pragma unroll
     for (int a = 0; a < NV; ++a) o[a] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int chunks = Dk >> 3;                                     // 16-byte pieces of a row
-
-    // this workgroup's share of the blocks of keys
-    int blk_first = key_lo >> 5, blk_end = (key_hi >> 5) + 1;
-    if (n_splits > 1) {
-        const int per = (blk_end - blk_first + n_splits - 1) / n_splits;
-        blk_first += (int)blockIdx.y * per;
-        blk_end = blk_first + per < blk_end ? blk_first + per : blk_end;
-    }
     // Staging: a thread keeps one key of the block (consecutive lanes take consecutive keys, so the
     // transposed copy's 2-byte stores fall into consecutive LDS words instead of one bank) and walks
     // that key's 16-byte pieces.  Where the key's row lies is looked up one block ahead, so the table
@@ -103,8 +164,13 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
             for (int e = 0; e < 8; ++e) Vt[(f + e) * LM_VT_LD + key] = v[e];
         }
     };
-    long long row_cur = blk_first < blk_end ? row_of(blk_first << 5) : -2;
+    if (roles) __syncthreads();                                     // the staging waves have looked up the share's rows
+    long long row_cur = (!roles && blk_first < blk_end) ? row_of(blk_first << 5) : -2;
     for (int blk0 = blk_first << 5; blk0 < (blk_end << 5); blk0 += 32) {
+      if (roles) {
+        __syncthreads();
+        __syncthreads();                                            // the staging waves have filled the block
+      } else {
         const long long row_next = blk0 + 32 < (blk_end << 5) ? row_of(blk0 + 32) : -2;
         __syncthreads();                                            // the last block's readers are done
         const bf16* src = kv_pages + (row_cur >= 0 ? row_cur : 0);
@@ -123,6 +189,7 @@ void attn_latent_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         if (tid < 32) kflag[key] = row_cur == -1;
         row_cur = row_next;
         __syncthreads();
+      }
         if (blk0 + 31 < wave_lo || blk0 > wave_hi) continue;        // nothing here for this wave's rows
 
         f32x4 s[2];
@@ -262,9 +329,14 @@ extern "C" int spite_attn_latent_mfma(const void* q, const void* kv_pages, void*
     // a wave for every 16 query rows, and enough waves that staging a block of 32 keys takes a thread
     // no more than about four 16-byte pieces (waves without rows only stage)
     int nw = (max_rows + 15) / 16;
-    const int stage_waves = (32 * (Dk / 8) + 255) / 256;
-    if (nw < stage_waves) nw = stage_waves < 8 ? stage_waves : 8;
-    const size_t sh = ((size_t)32 * (kq * 32 + 8) + (size_t)nv * 16 * LM_VT_LD) * sizeof(bf16) + 32 * sizeof(int);
+    const int pre = kq <= 6 ? 4 : (kq <= 10 ? 8 : LM_PRE);
+    const int fetch_waves = (Dk / 8 + 2 * pre - 1) / (2 * pre);         // staging waves (see the kernel)
+    if (nw + fetch_waves <= 8) nw += fetch_waves;
+    else {
+        const int stage_waves = (32 * (Dk / 8) + 255) / 256;
+        if (nw < stage_waves) nw = stage_waves < 8 ? stage_waves : 8;
+    }
+    const size_t sh = ((size_t)32 * (kq * 32 + 8) + (size_t)nv * 16 * LM_VT_LD) * sizeof(bf16) + (32 + LM_KROW_BLOCKS * 32) * sizeof(int);
 #define SP_LM(KQV, NVV) do { \
         auto kern = attn_latent_mfma_kernel<KQV, NVV>; \
         static bool allowed = false; \

@@ -717,7 +717,8 @@ def latent_splits(n_wg: int, longest: int) -> int:
     blocks of 32 keys (a workgroup's record is as large as what it reads of two or three such blocks)."""
     if n_wg <= 0:
         return 1
-    return max(1, min(-(-cu_count() // n_wg), -(-longest // 256), 256))
+    # (no fewer than keep a share within the 4,096 keys whose cache rows the staging waves look up ahead)
+    return max(1, min(-(-cu_count() // n_wg), -(-longest // 256), 256), min(-(-longest // 4096), 256))
 
 
 def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg, n_wg, max_rows, T, H, Dk, R, vis, span, scale,
