@@ -91,7 +91,7 @@ extern "C" int spite_latent_prepare(const void* qd, int ldq, const void* dkv, in
 // [first_visible(p), p] of the token's request; the value of a key is the first R elements of
 // its row.  Keys are walked in tiles of 64 that start at first_visible(p), so the order of every
 // sum depends on p alone.  Scores, maximum, sum and output are fp32, exp is the accurate one.
-#define LAT_MAX_V 8   // latents up to 512
+#define LAT_MAX_V 16  // latents up to 1,024
 
 template <typename T>
 __global__ __launch_bounds__(64)
