@@ -4,8 +4,8 @@ the host-side bookkeeping in the native cache manager.
 Layers are grouped by what they need: the same number of kv heads, head size and
 visibility (every key, the query's chunk, a window).  A group's pool is two tensors, keys
 ``[layers, pages, kv_heads, page_size, key width]`` and values, transposed,
-``[layers, pages, kv_heads, value width, page_size]`` (a mixer may ask for values of another
-width than its keys); a page is the same row range in every layer of the group, so one block
+``[layers, pages, value heads, value width, page_size]`` (a mixer may ask for values of another
+width than its keys, and for fewer value heads than key heads); a page is the same row range in every layer of the group, so one block
 table serves all of them.
 """
 from __future__ import annotations
@@ -33,7 +33,7 @@ class OutOfPages(CacheError):
 
 @dataclass
 class Group:
-    key: tuple                   # (kv heads, key width, visibility, span, value width)
+    key: tuple                   # (kv heads, key width, visibility, span, value width, value heads)
     cache_ids: List[int]
     n_pages: int
     k: Optional[torch.Tensor] = None     # [layers, pages, G, page_size, key width]
@@ -61,7 +61,8 @@ class PagedCache:
             if need is None or need.kv is None:
                 continue
             kv = need.kv
-            key = (kv.n_kv_heads, kv.head_dim, kv.visibility, kv.span if kv.visibility != "full" else 0, kv.value_dim)
+            key = (kv.n_kv_heads, kv.head_dim, kv.visibility, kv.span if kv.visibility != "full" else 0, kv.value_dim,
+                   kv.value_heads)
             if key not in by_key:
                 by_key[key] = len(self.groups)
                 self.groups.append(Group(key, [], 0, None))
@@ -99,9 +100,9 @@ class PagedCache:
         self.states: Dict[int, torch.Tensor] = {}
         if allocate:
             for g in self.groups:
-                G, kd, vd = g.key[0], g.key[1], g.key[4]
+                G, kd, vd, Gv = g.key[0], g.key[1], g.key[4], g.key[5]
                 g.k = torch.zeros((len(g.cache_ids), g.n_pages, G, self.page_size, kd), dtype=dtype, device=device)
-                g.v = torch.zeros((len(g.cache_ids), g.n_pages, G, vd, self.page_size), dtype=dtype, device=device)
+                g.v = torch.zeros((len(g.cache_ids), g.n_pages, Gv, vd, self.page_size), dtype=dtype, device=device)
             for cid, need in enumerate(needs):
                 if need is not None and need.state is not None:
                     self.states[cid] = torch.zeros((self.max_requests, *need.state.shape),

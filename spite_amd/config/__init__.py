@@ -2,5 +2,7 @@ from .llama4 import Llama4Config, RopeScaling, ConfigError
 from .registry import (register_architecture, architecture, registered_architectures, read_config,
                        UnknownArchitecture, Architecture)
 from .ravenex import RavenexConfig
+from .pefedra import PefedraConfig
 from . import llama4_spec  # noqa: F401  (registers Llama4ForCausalLM)
 from . import ravenex_spec  # noqa: F401  (registers Ravenex)
+from . import pefedra_spec  # noqa: F401  (registers Pefedra)

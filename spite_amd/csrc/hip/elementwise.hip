@@ -26,23 +26,24 @@ int sp_cu_count() {
 extern "C" int spite_cu_count() { return sp_cu_count(); }
 
 // ------------------------------------------------------------------ embedding
+// h[t] = table[ids[t]] * scale, in fp32 (scale 1: the row itself).
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ h, int d, int vocab) {
+                             float* __restrict__ h, int d, int vocab, float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     const bool ok = id >= 0 && id < vocab;
     const T* row = table + (size_t)(ok ? id : 0) * d;
     for (int c = threadIdx.x; c < d; c += blockDim.x)
-        h[(size_t)t * d + c] = ok ? to_f32<T>(row[c]) : 0.f;
+        h[(size_t)t * d + c] = ok ? to_f32<T>(row[c]) * scale : 0.f;
 }
 
 extern "C" int spite_embed(const int* ids, const void* table, int dtype, float* h, int T, int d,
-                           int vocab, hipStream_t st) {
+                           int vocab, float scale, hipStream_t st) {
     SP_REQUIRE(T >= 0 && d > 0 && vocab > 0, "embed: bad sizes T=%d d=%d vocab=%d", T, d, vocab);
     if (T == 0) return 0;
-    if (dtype == SP_F32) embed_kernel<float><<<T, 256, 0, st>>>(ids, (const float*)table, h, d, vocab);
-    else if (dtype == SP_BF16) embed_kernel<bf16><<<T, 256, 0, st>>>(ids, (const bf16*)table, h, d, vocab);
+    if (dtype == SP_F32) embed_kernel<float><<<T, 256, 0, st>>>(ids, (const float*)table, h, d, vocab, scale);
+    else if (dtype == SP_BF16) embed_kernel<bf16><<<T, 256, 0, st>>>(ids, (const bf16*)table, h, d, vocab, scale);
     else return sp_fail("embed: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("embed");
     return 0;

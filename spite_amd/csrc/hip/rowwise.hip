@@ -1,0 +1,90 @@
+// Small row-wise kernels: the token shift of a mixer's input, an activation applied in place,
+// and the two norms of a layer whose mixer and feed-forward read the same stream.
+#include "common.h"
+
+// ------------------------------------------------------------------ token shift
+// y[t] = x[t] + (x'[t] - x[t]) * w, with x'[t] the row of the token before t in its request: the
+// row t-1 of the step, or, for the first token of an entry, what the request's state row holds
+// (zeros for a request's first token: the state is cleared on admission).  The state then takes
+// the entry's last row.  The thread that reads an element of the state is the one that writes it,
+// after the read, so an entry of any length is safe; x and the state are fp32.
+template <typename TO>
+__global__ __launch_bounds__(256)
+void token_shift_kernel(const float* __restrict__ x, TO* __restrict__ y, const float* __restrict__ w,
+                        float* __restrict__ state, const int* __restrict__ seq_of_token,
+                        const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int d, int keep) {
+    const int t = blockIdx.x;
+    const int e = seq_of_token[t];
+    const int first = cu_seqlens[e], last = cu_seqlens[e + 1] - 1;
+    const float* xr = x + (size_t)t * d;
+    TO* yr = y + (size_t)t * d;
+    if (t != first) {
+        const float* xp = xr - d;
+        for (int c = threadIdx.x; c < d; c += 256) { const float a = xr[c]; yr[c] = from_f32<TO>(a + (xp[c] - a) * w[c]); }
+        return;
+    }
+    float* sr = state + (size_t)seq_slots[e] * d;
+    const float* xl = x + (size_t)last * d;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        const float a = xr[c];
+        yr[c] = from_f32<TO>(a + (sr[c] - a) * w[c]);
+        if (keep) sr[c] = xl[c];
+    }
+}
+
+extern "C" int spite_token_shift(const float* x, void* y, int y_dtype, const float* w, float* state,
+                                 const int* seq_of_token, const int* cu_seqlens, const int* seq_slots, int T, int d,
+                                 int keep, hipStream_t st) {
+    SP_REQUIRE(T >= 0 && d > 0, "token_shift: bad sizes T=%d d=%d", T, d);
+    if (T == 0) return 0;
+    if (y_dtype == SP_F32) token_shift_kernel<float><<<T, 256, 0, st>>>(x, (float*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
+    else if (y_dtype == SP_BF16) token_shift_kernel<bf16><<<T, 256, 0, st>>>(x, (bf16*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
+    else return sp_fail("token_shift: unknown dtype %d", y_dtype);
+    SP_LAUNCH_CHECK("token_shift");
+    return 0;
+}
+
+// ------------------------------------------------------------------ activation in place
+// SP_UNARY_GELU: 0.5 z (1 + erf(z / sqrt 2)); SP_UNARY_GELU_TANH; SP_UNARY_SILU.  fp32 inside.
+enum { SP_UNARY_GELU = 1, SP_UNARY_GELU_TANH = 2, SP_UNARY_SILU = 3 };
+__device__ __forceinline__ float sp_unary(float z, int act) {
+    if (act == SP_UNARY_GELU) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (act == SP_UNARY_GELU_TANH) return sp_gate_act(z, SP_ACT_GELU_TANH, false);
+    return sp_gate_act(z, SP_ACT_SILU, false);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256)
+void act_rows_kernel(T* __restrict__ x, size_t n, int act) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) x[i] = from_f32<T>(sp_unary(to_f32<T>(x[i]), act));
+}
+
+// eight bfloat16 a thread and step
+__global__ __launch_bounds__(256)
+void act_rows_bf16x8_kernel(bf16x8* __restrict__ x, size_t n8, int act) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
+        bf16x8 v = x[i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (bf16)sp_unary((float)v[e], act);
+        x[i] = v;
+    }
+}
+
+extern "C" int spite_act_rows(void* x, int dtype, size_t n, int act, hipStream_t st) {
+    SP_REQUIRE(act >= SP_UNARY_GELU && act <= SP_UNARY_SILU, "act_rows: activation %d", act);
+    if (n == 0) return 0;
+    if (dtype == SP_BF16 && n % 8 == 0 && ((uintptr_t)x & 15) == 0) {
+        const size_t n8 = n / 8;
+        const int blocks = (int)((n8 + 255) / 256 < 8192 ? (n8 + 255) / 256 : 8192);
+        act_rows_bf16x8_kernel<<<blocks, 256, 0, st>>>((bf16x8*)x, n8, act);
+    } else {
+        const int blocks = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+        if (dtype == SP_F32) act_rows_kernel<float><<<blocks, 256, 0, st>>>((float*)x, n, act);
+        else if (dtype == SP_BF16) act_rows_kernel<bf16><<<blocks, 256, 0, st>>>((bf16*)x, n, act);
+        else return sp_fail("act_rows: unknown dtype %d", dtype);
+    }
+    SP_LAUNCH_CHECK("act_rows");
+    return 0;
+}

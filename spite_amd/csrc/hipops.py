@@ -35,7 +35,7 @@ def lib():
         l.spite_hip_last_error.restype = c_char_p
         P, I, L, F = c_void_p, c_int, c_long, c_float
         sigs = {
-            "spite_embed": [P, P, I, P, I, I, I, P],
+            "spite_embed": [P, P, I, P, I, I, I, F, P],
             "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P, P, F, F, I, P],
             "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, I, P, P, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
@@ -63,6 +63,11 @@ def lib():
             "spite_router_topk": [P, P, P, P, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
+            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, P],
+            "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+            "spite_attn_finish": [P, I, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
+            "spite_token_shift": [P, P, I, P, P, P, P, P, I, I, I, P],
+            "spite_act_rows": [P, I, c_size_t, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -124,13 +129,13 @@ def _check(rc, what):
 
 
 # --------------------------------------------------------------------------------------------
-def embed(ids, table, h):
-    """h[t,:] = table[ids[t],:] as fp32.  ids int32 [T], table [V,d], h fp32 [T,d]."""
+def embed(ids, table, h, scale=1.0):
+    """h[t,:] = table[ids[t],:] * scale as fp32.  ids int32 [T], table [V,d], h fp32 [T,d]."""
     T, d = h.shape
     if ids.numel() != T or table.shape[1] != d:
         raise KernelError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, h {tuple(h.shape)}")
     _check(lib().spite_embed(_ptr(ids, "ids", torch.int32), _ptr(table, "table"), dtype_code(table.dtype),
-                             _ptr(h, "h", torch.float32), T, d, table.shape[0], _stream()), "embed")
+                             _ptr(h, "h", torch.float32), T, d, table.shape[0], float(scale), _stream()), "embed")
 
 
 def add_rmsnorm_can_project(d: int) -> bool:
@@ -742,3 +747,109 @@ def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg,
         block_table.shape[1], _ptr(wg, "wg", torch.int32), int(n_wg), int(max_rows), H, Dk, R, kv_pages.shape[2],
         VIS[vis], int(span or 0), float(scale), _ptr(scratch, "scratch", torch.float32) if n_splits > 1 else None,
         n_splits, T * H, _stream()), "latent attention (MFMA)")
+
+
+# -------------------------------------------------------------------------------------------- keys and values of unequal shape
+def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D, Vd, page_size, *, bias=None,
+                norm_q=None, norm_k=None, eps=0.0, inv_freq=None, rot=0, inv_freq_v=None, write_kv=True,
+                k_tiled=False, v_tiled=False):
+    """Between a fused projection and the cache (see attn_wide.hip).  qkv: rows that begin with
+    [HQ*D | GK*D | GV*Vd] (further columns are left alone); ``bias`` fp32 over those; ``norm_q`` /
+    ``norm_k`` (fp32 [HQ*D], [GK*D]): weights of an RMS norm over the whole q and the whole k part;
+    ``inv_freq`` (fp32 [rot/2]): the first ``rot`` elements of every q and k head turn in pairs
+    (i, i + rot/2); ``inv_freq_v`` (fp32 [Vd/2]): the values turn in pairs (m, m + Vd/2).  q_out
+    [T, HQ*D]; key pages [pages, GK, page_size, D]; value pages [pages, GV, Vd, page_size]."""
+    T = qkv.shape[0]
+    n = (HQ + GK) * D + GV * Vd
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n:
+        raise KernelError(f"qkv_prepare: rows {tuple(qkv.shape)} for HQ={HQ} GK={GK} GV={GV} D={D} Vd={Vd}")
+    if q_out.numel() < T * HQ * D or positions.numel() < T:
+        raise KernelError("qkv_prepare: q_out or positions too small")
+    if write_kv:
+        if slot_map is None or slot_map.numel() < T:
+            raise KernelError("qkv_prepare: slot map too small")
+        if tuple(k_pages.shape[1:]) != (GK, page_size, D) or tuple(v_pages.shape[1:]) != (GV, Vd, page_size) \
+                or k_pages.shape[0] != v_pages.shape[0]:
+            raise KernelError(f"qkv_prepare: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
+                              f"GK={GK} GV={GV} page={page_size} D={D} Vd={Vd}")
+    for name, t, size in (("bias", bias, n), ("norm_q", norm_q, HQ * D), ("norm_k", norm_k, GK * D),
+                          ("inv_freq", inv_freq, rot // 2), ("inv_freq_v", inv_freq_v, Vd // 2)):
+        if t is not None and t.numel() != size:
+            raise KernelError(f"qkv_prepare: {name} of {t.numel()} values, expected {size}")
+    if rot and inv_freq is None:
+        raise KernelError("qkv_prepare: rotation needs a frequency table")
+    dt = qkv.dtype
+    _check(lib().spite_qkv_prepare(
+        qkv.data_ptr() if qkv.is_cuda else _ptr(qkv, "qkv"), qkv.stride(0), dtype_code(dt), _ptr(bias, "bias", torch.float32, True),
+        _ptr(norm_q, "norm_q", torch.float32, True), _ptr(norm_k, "norm_k", torch.float32, True), float(eps),
+        _ptr(q_out, "q_out", dt), _ptr(k_pages, "k_pages", dt, not write_kv), _ptr(v_pages, "v_pages", dt, not write_kv),
+        _ptr(positions, "positions", torch.int32), _ptr(slot_map, "slot_map", torch.int32) if write_kv else None,
+        _ptr(inv_freq, "inv_freq", torch.float32, True), int(rot), _ptr(inv_freq_v, "inv_freq_v", torch.float32, True),
+        T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), _stream()), "qkv_prepare")
+
+
+def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, HQ, GK, GV, D, Vd, page_size, vis, span,
+              scale, k_tiled=False, v_tiled=False):
+    """Attention over the paged cache with keys of D and values of Vd elements, HQ query heads over
+    GK key heads over GV value heads (query head h: key head h // (HQ/GK), value head of that % GV);
+    any mix of portions and single tokens.  q [T, HQ*D]; out [T, HQ*Vd] in q's dtype or fp32."""
+    if q.numel() < T * HQ * D or out.numel() < T * HQ * Vd:
+        raise KernelError("attention: q or out too small")
+    if tuple(k_pages.shape[1:]) != (GK, page_size, D) or tuple(v_pages.shape[1:]) != (GV, Vd, page_size) \
+            or k_pages.shape[0] != v_pages.shape[0]:
+        raise KernelError(f"attention: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
+                          f"GK={GK} GV={GV} page={page_size} D={D} Vd={Vd}")
+    if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
+        raise KernelError("attention: metadata too small")
+    dt = q.dtype
+    _check(lib().spite_attn_wide(
+        _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out"), dtype_code(dt),
+        dtype_code(out.dtype), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
+        _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, HQ, GK, GV, D, Vd, page_size,
+        VIS[vis], int(span or 0), float(scale), int(bool(k_tiled)), int(bool(v_tiled)), _stream()), "attention")
+
+
+def attn_finish(a, out, positions, H, Vd, *, maps=1, lam=0.0, eps=0.0, post=1.0, inv_freq_v=None, gate=None):
+    """From the attention's result to the output projection's operand (see attn_wide.hip).  a
+    [T, maps*H*Vd] (map by map), out [T, H*Vd].  ``maps`` = 2: a1 - lam * a2, divided by its root mean
+    square over the head (``eps``), times ``post``.  ``inv_freq_v``: pairs (m, m + Vd/2) turn back by
+    the position.  ``gate``: a [T, >= H] view (rows may lie apart) of logits, one per head, whose
+    sigmoid multiplies the head."""
+    T = out.shape[0]
+    if a.numel() < T * maps * H * Vd or out.numel() < T * H * Vd:
+        raise KernelError("attn_finish: input or output too small")
+    ldg = 0
+    if gate is not None:
+        if gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[1] < H or gate.shape[0] < T or gate.dtype != out.dtype:
+            raise KernelError(f"attn_finish: gate {tuple(gate.shape)} {gate.dtype} for {H} heads")
+        ldg = gate.stride(0)
+    if inv_freq_v is not None and inv_freq_v.numel() != Vd // 2:
+        raise KernelError("attn_finish: frequency table does not match the values")
+    _check(lib().spite_attn_finish(
+        _ptr(a, "a"), dtype_code(a.dtype), _ptr(out, "out"), dtype_code(out.dtype), _ptr(positions, "positions", torch.int32),
+        _ptr(inv_freq_v, "inv_freq_v", torch.float32, True), gate.data_ptr() if gate is not None else None, ldg,
+        T, H, Vd, int(maps), float(lam), float(eps), float(post), _stream()), "attn_finish")
+
+
+def token_shift(x, y, w, state, seq_of_token, cu_seqlens, seq_slots, keep=True):
+    """y[t] = x[t] + (x[t-1] - x[t]) * w within a request; the first token of an entry takes the
+    request's state row for x[t-1], which then receives the entry's last row (``keep``).  x fp32
+    [T, d], y [T, d], w fp32 [d], state fp32 [slots, d]."""
+    T, d = x.shape
+    if y.shape != x.shape or w.numel() != d or state.dim() != 2 or state.shape[1] != d or seq_of_token.numel() < T:
+        raise KernelError(f"token_shift: x {tuple(x.shape)}, y {tuple(y.shape)}, state {tuple(state.shape)}")
+    _check(lib().spite_token_shift(
+        _ptr(x, "x", torch.float32), _ptr(y, "y"), dtype_code(y.dtype), _ptr(w, "w", torch.float32),
+        _ptr(state, "state", torch.float32), _ptr(seq_of_token, "seq_of_token", torch.int32),
+        _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32), T, d, int(bool(keep)),
+        _stream()), "token_shift")
+
+
+UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def act_rows(x, act):
+    """x = act(x) in place: ``gelu`` (the erf form), ``gelu_tanh`` or ``silu``; fp32 inside."""
+    if act not in UNARY_ACTS:
+        raise KernelError(f"act_rows: activation {act!r} (known: {sorted(UNARY_ACTS)})")
+    _check(lib().spite_act_rows(_ptr(x, "x"), dtype_code(x.dtype), x.numel(), UNARY_ACTS[act], _stream()), "act_rows")

@@ -34,10 +34,16 @@ class KVNeed:
     visibility: str = "full"          # "full" | "chunk" | "window"
     span: int = 0                     # chunk size or window
     v_head_dim: Optional[int] = None  # width of a value where it differs from a key's (the pool's two halves are sized apart)
+    n_v_heads: Optional[int] = None   # value heads where they are fewer than the key heads (several key heads, the
+                                      # score maps of one head, share a value head)
 
     @property
     def value_dim(self) -> int:
         return self.head_dim if self.v_head_dim is None else int(self.v_head_dim)
+
+    @property
+    def value_heads(self) -> int:
+        return self.n_kv_heads if self.n_v_heads is None else int(self.n_v_heads)
 
 
 @dataclass(frozen=True)
@@ -190,6 +196,19 @@ class SideInput(Part):
         raise NotImplementedError
 
 
+class InputShift(Part):
+    """Something that changes what a mixer reads from the normed stream, with a state row per
+    request of its own (what it has to remember of the request's earlier tokens)."""
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, x32, out, ctx, state) -> None:
+        """x32 fp32 [T, d] (the normed stream) -> out [T, d] in the run's dtype; ``state`` is the
+        ``[max_requests, ...]`` tensor that ``state_need`` asked for."""
+        raise NotImplementedError
+
+
 class Embedding(Part):
     #: the table [V, d] after loading, for a head that is tied to it (None if there is none)
     table = None
@@ -290,6 +309,7 @@ def step_array_builder(name: str) -> Callable:
 # ----------------------------------------------------------------------------- registries
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {
     "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {}, "side": {},
+    "shift": {},
 }
 
 

@@ -1,4 +1,4 @@
-"""Arrangement of a layer: pre-norm residual block,
+"""Arrangements of a layer.  ``prenorm``: pre-norm residual block,
 h += mixer(norm1(h)); h += ffn(norm2(h)) (crates/spite-models/src/llama/llama4.rs:126-127,
 202-211, 272-274).  The additions are folded into the norm that follows them: a block hands
 its last increments to the next block (or the final norm) instead of adding them itself."""
@@ -149,4 +149,83 @@ class SandwichBlock(Block):
             pend = (self.norm2b.as_increment(f[0], self.mult),)
         if self.side is not None:
             pend = tuple(self.side.forward(h, pend, ctx))
+        state["pending"] = pend
+
+
+@register("block", "parallel")
+class ParallelBlock(Block):
+    """Mixer and feed-forward read the same stream, each through a norm of its own, and their
+    results join it together:  h += mixer(shift(norm1(h))) + ffn(norm2(h)).  ``spec.extra["shift"]``
+    (a PartSpec of category ``shift``, optional) stands between the first norm and the mixer and
+    keeps a state row per request; the feed-forward may be missing.  Both results are handed to the
+    next block, whose first norm adds them."""
+    graph_safe = True
+
+    def __init__(self, env, spec):
+        self.env = env
+        self.norm1 = build_part("norm", spec.norm1, env)
+        self.mixer = build_part("mixer", spec.mixer, env)
+        self.children = [("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer)]
+        self.shift = self.norm2 = self.ffn = None
+        sh = spec.extra.get("shift")
+        if sh is not None:
+            self.shift = build_part("shift", sh, env)
+            self.children.append(("shift", self.shift, sh))
+        if spec.ffn is not None:
+            self.norm2 = build_part("norm", spec.norm2, env)
+            self.ffn = build_part("ffn", spec.ffn, env)
+            self.children += [("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn)]
+        self.children = tuple(self.children)
+        self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
+        self.step_arrays = tuple(sorted({a for _, part, _ in self.children for a in part.step_arrays}))
+
+    def cache_needs(self):
+        needs = {"mixer": self.mixer.cache_need()}
+        if self.shift is not None and self.shift.state_need() is not None:
+            from .base import CacheNeed
+            needs["shift"] = CacheNeed(state=self.shift.state_need())
+        return needs
+
+    def forward(self, h, pending, ctx, cache):
+        state = {"h": h, "pending": pending}
+        for _, stage in self.stages():
+            stage(state, ctx, cache)
+        return state["pending"]
+
+    def stages(self):
+        first = all(p.graph_safe for p in (self.norm1, self.shift, self.norm2) if p is not None)
+        return [(first, self._stage_norms), (self.mixer.graph_safe, self._stage_mixer),
+                (self.ffn is None or self.ffn.graph_safe, self._stage_ffn)]
+
+    def _stage_norms(self, state, ctx, cache):
+        h, ws = state["h"], ctx.ws
+        T, d = h.shape
+        d1, d2 = two_increments(h, state["pending"])
+        if self.shift is not None:
+            # the shift blends fp32 rows; the mixer's input takes the run's dtype after it
+            n32 = ws.take((T, d), torch.float32)
+            self.norm1.forward(h, None, d1=d1, d2=d2, out32=n32)
+            x = ws.take((T, d), self.env.dtype)
+            self.shift.forward(n32, x, ctx, cache["shift"].state)        # a block with a shift has two caches, by name
+        else:
+            x = ws.take((T, d), self.env.dtype)
+            self.norm1.forward(h, x, d1=d1, d2=d2)
+        state["mixer_in"] = x
+        if self.ffn is not None:
+            # the same stream (the increments are in it now) through the second norm
+            n2 = ws.take((T, d), self.env.dtype)
+            n2_32 = None
+            if self.ffn.wants_f32_input:
+                n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
+            self.norm2.forward(h, n2, out32=None if n2_32 is n2 else n2_32, write_h=False)
+            state["ffn_in"] = (n2, n2_32)
+
+    def _stage_mixer(self, state, ctx, cache):
+        state["mixed"] = self.mixer.forward(state.pop("mixer_in"), ctx, cache["mixer"] if isinstance(cache, dict) else cache)
+
+    def _stage_ffn(self, state, ctx, cache):
+        pend = (state.pop("mixed"),)
+        if self.ffn is not None:
+            n2, n2_32 = state.pop("ffn_in")
+            pend += tuple(self.ffn.forward(n2, n2_32, ctx))
         state["pending"] = pend

@@ -1,7 +1,7 @@
 """The two ends of a model: token ids in, logits out.
 
 ``token_table`` (crates/spite-models/src/llama/llama4.rs:118-119): row ``id`` of the table as
-the residual stream's first value, in fp32.
+the residual stream's first value, in fp32, times ``scale`` if the architecture has one.
 ``linear_head`` (llama4.rs:277-279): logits = W . (normed last hidden state), W ``[V, d]``;
 tied, it reads the embedding's table.  Another architecture's embedding scale, logit cap or
 bias is another kind registered under these categories, not a change to the model class.
@@ -17,8 +17,9 @@ from ..csrc import hipops
 class TokenTable(Embedding):
     graph_safe = True
 
-    def __init__(self, env, vocab_size: int, width: int):
-        self.V, self.d = int(vocab_size), int(width)
+    def __init__(self, env, vocab_size: int, width: int, scale: float = 1.0):
+        """``scale``: a constant on every row as it enters the stream (fp32)."""
+        self.V, self.d, self.scale = int(vocab_size), int(width), float(scale)
         self.table = None
 
     def params(self):
@@ -28,7 +29,7 @@ class TokenTable(Embedding):
         self.table = tensors["weight"].contiguous()
 
     def forward(self, token_ids, h, ctx):
-        hipops.embed(token_ids, self.table, h)
+        hipops.embed(token_ids, self.table, h, self.scale)
 
 
 @register("head", "linear_head")

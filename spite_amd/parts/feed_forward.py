@@ -3,6 +3,9 @@
 ``dense_glu`` (crates/spite-models/src/llama/llama4.rs:257-271):
 y = W_down . (silu(W_gate . x) * (W_up . x)).
 
+``dense_mlp``: y = W_down . act(W_up . x), no gate; ``activation``: ``gelu`` (the erf form),
+``gelu_tanh`` or ``silu``, applied in fp32 to the up projection's rows.
+
 ``moe_top1_sigmoid`` (crates/spite-models/src/moe.rs:87-194, llama4.rs:212-256): router
 logits W_r . x in fp32; the expert with the largest logit (lowest index on ties); its
 *input* is x * sigmoid(logit), its output is not weighted; a shared expert on the unscaled
@@ -60,6 +63,36 @@ class DenseGLU(FeedForward):
         linear(x, self.w_gate_up, act, glu=self.activation, ws=ctx.ws)
         y = ctx.ws.take((T, self.d), torch.float32)
         linear(act, self.w_down, y, ws=ctx.ws)
+        return (y,)
+
+
+@register("ffn", "dense_mlp")
+class DenseMLP(FeedForward):
+    graph_safe = True
+
+    def __init__(self, env, hidden_size, intermediate_size, activation="gelu"):
+        self.d, self.F = int(hidden_size), int(intermediate_size)
+        if activation not in hipops.UNARY_ACTS:
+            raise ValueError(f"dense_mlp: activation {activation!r} (known: {sorted(hipops.UNARY_ACTS)})")
+        self.activation = activation
+        self.w_up = self.w_down = None
+
+    def params(self):
+        return {"up_proj": ParamSpec((self.F, self.d)), "down_proj": ParamSpec((self.d, self.F))}
+
+    def load(self, t):
+        self.w_up, self.w_down = Weight(t["up_proj"]), Weight(t["down_proj"])
+
+    def slow_paths(self, page_size):
+        return self.w_up.slow_reason("up projection") + self.w_down.slow_reason("down projection")
+
+    def forward(self, x, x32, ctx, projected=None):
+        T = x.shape[0]
+        u = ctx.ws.take((T, self.F), x.dtype)
+        linear(x, self.w_up, u, ws=ctx.ws)
+        hipops.act_rows(u, self.activation)
+        y = ctx.ws.take((T, self.d), torch.float32)
+        linear(u, self.w_down, y, ws=ctx.ws)
         return (y,)
 
 

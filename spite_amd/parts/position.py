@@ -4,7 +4,8 @@
 (crates/spite-rope/src/lib.rs:78-92; half-split pairs (i, i+hd/2) as there, or adjacent
 pairs), f_i = theta^(-2i/hd), optionally rescaled once at load by the ``llama3`` rule
 (wavelength L = 2*pi/f: L < orig/high keeps f; L > orig/low gives f/factor; between, the
-blend (1-s)*f/factor + s*f with s = (orig/L - low)/(high - low)).  The table is computed in
+blend (1-s)*f/factor + s*f with s = (orig/L - low)/(high - low)) or by the ``linear`` rule
+(every f divided by ``factor``: positions counted in units of ``factor`` tokens).  The table is computed in
 float64 and stored as fp32; angle and rotation are fp32 in the kernel.
 
 ``none``: no position information (NoPE layers).
@@ -23,7 +24,9 @@ def inv_frequencies(head_dim: int, theta: float, scaling=None):
     out = []
     for i in range(half):
         f = 1.0 / (float(theta) ** (2.0 * i / head_dim))
-        if scaling is not None:
+        if scaling is not None and scaling.get("rope_type", "llama3") == "linear":
+            f = f / float(scaling["factor"])
+        elif scaling is not None:
             factor, low, high, orig = (float(scaling["factor"]), float(scaling["low_freq_factor"]),
                                        float(scaling["high_freq_factor"]),
                                        float(scaling["original_max_position_embeddings"]))
@@ -51,7 +54,7 @@ class Rotary(PositionEncoding):
             raise ValueError(f"rotary: head size {head_dim} and rotating part {rot} must be even, the part within the head")
         if pairing not in ("half", "adjacent"):
             raise ValueError(f"rotary: pairing {pairing!r}")
-        if scaling is not None and scaling.get("rope_type", "llama3") != "llama3":
+        if scaling is not None and scaling.get("rope_type", "llama3") not in ("llama3", "linear"):
             raise ValueError(f"rotary: scaling of type {scaling.get('rope_type')!r} is not known")
         self.adjacent = pairing == "adjacent"
         self.rotary_dim = rot

@@ -1,0 +1,211 @@
+"""Attention whose keys and values differ in shape, with the options that stand around it.
+
+``wide_attention`` is grouped-query attention over the paged cache, H query heads on G kv heads,
+keys and queries ``key_dim`` wide, values ``value_dim`` wide, with, each as an option:
+
+* ``bias``: q, k and v projections with biases (``q_bias``, ``k_bias``, ``v_bias``);
+* ``projection_norm``: an RMS norm over the whole q projection and over the whole k projection
+  (all heads at once, weights ``q_norm`` [H*key_dim] and ``k_norm`` [G*key_dim]) before the rotation;
+* the position encoding of q and k (a ``position`` part; its first ``rotary_dim`` elements turn);
+* ``value_position``: the values turn by their own position before they are cached, over all of
+  ``value_dim``, and every head's result is turned back by the query's position: value j reaches
+  query i turned by j - i;
+* ``maps`` = 2, differential attention: every head has two queries and two keys (rows laid out
+  head by head as [map 1 | map 2]); each map is a softmax attention of its own over the same
+  values, and the head's result is ``a1 - lambda * a2`` divided by its root mean square over the
+  head's values, times ``1 - diff``; lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff is one number
+  of the layer, formed from four vectors of the checkpoint when it is loaded;
+* ``head_gate``: head h's result times sigmoid(W_g x)_h (``gate_proj`` [H, d]), before the output
+  projection.
+
+Inside, two maps are 2H query heads over 2G key heads over G value heads: the projections' rows
+are reordered map by map when they are loaded, so that query head m*H + h reads key head
+m*G + g and value head g.  Scores, softmax, the sums over the values, norms, angles and the gate's
+sigmoid are fp32 in both dtypes.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .base import Mixer, ParamSpec, CacheNeed, KVNeed, register, build as build_part
+from .attention import TAIL
+from .linear import linear, Weight
+from ..csrc import hipops
+
+
+@register("mixer", "wide_attention")
+class WideAttention(Mixer):
+    graph_safe = True
+    step_arrays = (TAIL,)
+
+    def __init__(self, env, hidden_size, n_heads, n_kv_heads, key_dim, value_dim, scale, position=None,
+                 value_position=None, visibility="full", span=0, bias=False, projection_norm=False, norm_eps=1e-5,
+                 maps=1, diff=0.0, head_gate=False):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"wide_attention: {n_heads} heads over {n_kv_heads} kv heads")
+        if visibility not in hipops.VIS:
+            raise ValueError(f"wide_attention: visibility {visibility!r} (known: {sorted(hipops.VIS)})")
+        if visibility != "full" and span < 1:
+            raise ValueError(f"wide_attention: {visibility} of size {span}")
+        if maps not in (1, 2):
+            raise ValueError(f"wide_attention: {maps} score maps a head")
+        if maps == 2 and (value_position is not None or head_gate):
+            raise ValueError("wide_attention: two score maps go with neither turned values nor a head gate")
+        self.env = env
+        self.d, self.H, self.G = int(hidden_size), int(n_heads), int(n_kv_heads)
+        self.D, self.Vd, self.maps = int(key_dim), int(value_dim), int(maps)
+        self.scale, self.diff, self.eps = float(scale), float(diff), float(norm_eps)
+        self.visibility, self.span = visibility, int(span or 0)
+        self.bias, self.projection_norm, self.head_gate = bool(bias), bool(projection_norm), bool(head_gate)
+        self.position = build_part("position", position, env) if position is not None else None
+        self.value_position = build_part("position", value_position, env) if value_position is not None else None
+        for pe in (self.position, self.value_position):
+            if pe is not None and (not pe.fused or pe.kernel_args().get("adjacent")):
+                raise ValueError("wide_attention: the position encoding must be a rotation in halves")
+        self.HQ, self.GK = self.H * self.maps, self.G * self.maps
+        self.n_qkv = (self.HQ + self.GK) * self.D + self.G * self.Vd
+        self.w_in = self.wo = self.b_in = self.w_qnorm = self.w_knorm = None
+        self.inv_freq = self.inv_freq_v = None
+        self.rot = 0
+        self.lam = 0.0
+
+    # ------------------------------------------------------------------ tensors
+    def params(self):
+        d, H, G, D, Vd, m = self.d, self.H, self.G, self.D, self.Vd, self.maps
+        p = {"q_proj": ParamSpec((H * m * D, d)), "k_proj": ParamSpec((G * m * D, d)), "v_proj": ParamSpec((G * Vd, d)),
+             "o_proj": ParamSpec((d, H * Vd))}
+        if self.bias:
+            p.update({"q_bias": ParamSpec((H * m * D,), kind="vector", init="normal"),
+                      "k_bias": ParamSpec((G * m * D,), kind="vector", init="normal"),
+                      "v_bias": ParamSpec((G * Vd,), kind="vector", init="normal")})
+        if self.projection_norm:
+            p.update({"q_norm": ParamSpec((H * D,), kind="vector", init="ones"),
+                      "k_norm": ParamSpec((G * D,), kind="vector", init="ones")})
+        if self.maps == 2:
+            p.update({k: ParamSpec((D,), kind="vector", init="normal") for k in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2")})
+        if self.head_gate:
+            p["gate_proj"] = ParamSpec((H, d))
+        return p
+
+    def _by_map(self, t, heads):
+        """Rows [head][map][D] of a projection (or bias) reordered to [map][head][D]."""
+        if self.maps == 1:
+            return t
+        rest = t.shape[1:]
+        return t.reshape(heads, self.maps, self.D, *rest).transpose(0, 1).reshape(heads * self.maps * self.D, *rest).contiguous()
+
+    def load(self, t):
+        H, G = self.H, self.G
+        mats = [self._by_map(t["q_proj"], H), self._by_map(t["k_proj"], G), t["v_proj"]]
+        if self.head_gate:
+            mats.append(t["gate_proj"])
+        dts = {m.dtype for m in mats}
+        dt = torch.float32 if len(dts) > 1 else dts.pop()
+        w = torch.cat([m.to(dt) for m in mats], dim=0)
+        pad = -w.shape[0] % 16           # whole bands of 16 rows: the weight can be kept in operand order
+        if pad:
+            w = torch.cat([w, torch.zeros((pad, w.shape[1]), dtype=dt, device=w.device)], dim=0)
+        self.n_in = w.shape[0]
+        self.w_in = Weight(w)
+        self.wo = Weight(t["o_proj"])
+        if self.bias:
+            self.b_in = torch.cat([self._by_map(t["q_bias"], H), self._by_map(t["k_bias"], G), t["v_bias"]]).float().contiguous()
+        if self.projection_norm:
+            self.w_qnorm, self.w_knorm = t["q_norm"].float().contiguous(), t["k_norm"].float().contiguous()
+        if self.maps == 2:
+            dot = lambda a, b: float((t[a].double() * t[b].double()).sum())
+            self.lam = math.exp(dot("lambda_q1", "lambda_k1")) - math.exp(dot("lambda_q2", "lambda_k2")) + self.diff
+        if self.position is not None:
+            ka = self.position.kernel_args()
+            if ka["use_rope"]:
+                self.inv_freq, self.rot = ka["inv_freq"], int(ka.get("rotary_dim") or self.D)
+                if self.rot > self.D:
+                    raise ValueError(f"wide_attention: {self.rot} turning elements in heads of {self.D}")
+        if self.value_position is not None:
+            ka = self.value_position.kernel_args()
+            if int(ka.get("rotary_dim") or self.Vd) != self.Vd or self.Vd % 2:
+                raise ValueError("wide_attention: the values' rotation covers the whole (even) value width")
+            self.inv_freq_v = ka["inv_freq"]
+
+    def slow_paths(self, page_size):
+        notes = []
+        if self.env.dtype == torch.bfloat16:
+            if not self._mfma(page_size):
+                notes.append(f"attention runs on plain FMAs: keys of {self.D} and values of {self.Vd} elements, pages of "
+                             f"{page_size} (the MFMA kernels take equal widths of 64 or 128 and pages in multiples of 32)")
+            for name, w in (("q/k/v projection", self.w_in), ("output projection", self.wo)):
+                if w is not None:
+                    notes += w.slow_reason(name)
+        return notes
+
+    def cache_need(self):
+        return CacheNeed(kv=KVNeed(self.GK, self.D, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G))
+
+    def _mfma(self, page_size):
+        return (self.env.dtype == torch.bfloat16 and self.D == self.Vd and self.D in (64, 128) and page_size % 32 == 0
+                and self.HQ // self.GK <= 16 and self.maps == 1)
+
+    # ------------------------------------------------------------------ the step
+    def _decode(self, q, o, ctx, cache, T):
+        HQ, GK, D = self.HQ, self.GK, self.D
+        longest = cache.block_table.shape[1] * cache.page_size
+        if self.visibility != "full":
+            longest = min(longest, self.span + 32)
+        blocks = -(-longest // 32)
+        n_splits = max(1, min(-(-2 * hipops.cu_count() // (T * GK)), -(-blocks // 8), 256))
+        scratch = ctx.ws.take((hipops.attn_decode_workspace(T, HQ, D, n_splits) // 4,), torch.float32)
+        hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
+                           cache.block_table, T, HQ, GK, D, cache.page_size, self.visibility, self.span,
+                           self.scale, n_splits)
+
+    def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
+        HQ, GK, D = self.HQ, self.GK, self.D
+        counts, starts = ctx.host.counts[lead:], ctx.host.starts[lead:]
+        longest = int((starts + counts).max())
+        if self.visibility != "full":
+            longest = min(longest, self.span + int(counts.max()))
+        n_splits = hipops.attn_prefill_splits(counts, HQ, GK, longest)
+        scratch = None
+        if n_splits > 1:
+            scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, HQ, GK, D, n_splits) // 4,), torch.float32)
+        hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
+                            cache.block_table[lead:], HQ, GK, D, cache.page_size, self.visibility, self.span, self.scale,
+                            n_splits=n_splits, scratch=scratch)
+
+    def forward(self, x, ctx, cache):
+        T, ws = x.shape[0], ctx.ws
+        H, G, HQ, GK, D, Vd = self.H, self.G, self.HQ, self.GK, self.D, self.Vd
+        proj = ws.take((T, self.n_in), x.dtype)
+        linear(x, self.w_in, proj, ws=ws)
+        q = ws.take((T, HQ * D), x.dtype)
+        hipops.qkv_prepare(proj, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, HQ, GK, G, D, Vd,
+                           cache.page_size, bias=self.b_in, norm_q=self.w_qnorm, norm_k=self.w_knorm, eps=self.eps,
+                           inv_freq=self.inv_freq, rot=self.rot, inv_freq_v=self.inv_freq_v, write_kv=cache.write,
+                           k_tiled=cache.tiled, v_tiled=cache.tiled)
+        if cache.tiled and self._mfma(cache.page_size):
+            a = ws.take((T, HQ * Vd), x.dtype)
+            cu_tail, lead = ctx.derived[TAIL]
+            if ctx.decode_only:
+                self._decode(q, a, ctx, cache, T)
+            else:
+                if lead:                   # decoded tokens of other requests beside prompt portions
+                    self._decode(q, a, ctx, cache, lead)
+                self._prefill(q[lead:], a[lead:], ctx, cache, lead, cu_tail if lead else ctx.cu_seqlens)
+        else:
+            # two maps meet in a difference: keep them in fp32 until then
+            a = ws.take((T, HQ * Vd), torch.float32 if self.maps == 2 else x.dtype)
+            hipops.attn_wide(q, cache.k_pages, cache.v_pages, a, ctx.positions, ctx.seq_of_token, cache.block_table,
+                             T, HQ, GK, G, D, Vd, cache.page_size, self.visibility, self.span, self.scale,
+                             k_tiled=cache.tiled, v_tiled=cache.tiled)
+        if self.maps == 2 or self.inv_freq_v is not None or self.head_gate:
+            o = ws.take((T, H * Vd), x.dtype)
+            gate = proj[:, self.n_qkv:self.n_qkv + H] if self.head_gate else None
+            hipops.attn_finish(a, o, ctx.positions, H, Vd, maps=self.maps, lam=self.lam, eps=self.eps,
+                               post=1.0 - self.diff, inv_freq_v=self.inv_freq_v, gate=gate)
+        else:
+            o = a
+        out = ws.take((T, self.d), torch.float32)
+        linear(o, self.wo, out, ws=ws)
+        return out
