@@ -415,9 +415,10 @@ def kv_operand_order(k_pages, v_pages):
     k = k_pages.reshape(n, G, ps // 32, 4, 2, 4, hd // 32, 4, 8)          # b, a, tt, i, cc, q, e
     k = k.permute(0, 1, 2, 4, 6, 7, 3, 5, 8)                                # b, tt, cc, q, a, i, e
     # head element c = 16dt + r, key offset = 32b + 8q + e
-    v = v_pages.reshape(n, G, hd // 16, 16, ps // 32, 4, 8)                # dt, r, b, q, e
+    Gv = v_pages.shape[1]                                                   # value heads may be fewer than key heads
+    v = v_pages.reshape(n, Gv, hd // 16, 16, ps // 32, 4, 8)               # dt, r, b, q, e
     v = v.permute(0, 1, 4, 2, 5, 3, 6)                                      # b, dt, q, r, e
-    return k.contiguous().view(n, G, ps, hd), v.contiguous().view(n, G, hd, ps)
+    return k.contiguous().view(n, G, ps, hd), v.contiguous().view(n, Gv, hd, ps)
 
 
 def attn_decode_workspace(T, H, hd, n_splits) -> int:
@@ -826,7 +827,8 @@ def attn_finish(a, out, positions, H, Vd, *, maps=1, lam=0.0, eps=0.0, post=1.0,
     if inv_freq_v is not None and inv_freq_v.numel() != Vd // 2:
         raise KernelError("attn_finish: frequency table does not match the values")
     _check(lib().spite_attn_finish(
-        _ptr(a, "a"), dtype_code(a.dtype), _ptr(out, "out"), dtype_code(out.dtype), _ptr(positions, "positions", torch.int32),
+        _ptr(a, "a"), dtype_code(a.dtype), _ptr(out, "out"), dtype_code(out.dtype),
+        _ptr(positions, "positions", torch.int32, inv_freq_v is None),
         _ptr(inv_freq_v, "inv_freq_v", torch.float32, True), gate.data_ptr() if gate is not None else None, ldg,
         T, H, Vd, int(maps), float(lam), float(eps), float(post), _stream()), "attn_finish")
 
