@@ -31,7 +31,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
                         int span, float scale_log2e, float cap_ratio, int n_splits,
-                        const float* __restrict__ slopes, float inv_scale) {
+                        const float* __restrict__ slopes, float inv_scale, int Gv) {
     constexpr int NC = HD / 32;      // 32-wide chunks of the head for the score product
     constexpr int ND = HD / 16;      // 16-row tiles of the output
     constexpr int ROW = HD + 2;      // partial record: output, max, sum
@@ -70,7 +70,8 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         const size_t pg = (size_t)(page < 0 ? 0 : page) * G + g;
         const int blk = off0 >> 5;                                   // the block of 32 keys inside the page
         const bf16* kbase = k_pages + pg * ps * HD + (size_t)blk * 2 * NC * 512 + lane * 8;
-        const bf16* vbase = v_pages + pg * HD * ps + (size_t)blk * ND * 512 + lane * 8;
+        // (value heads may be fewer than key heads: key head g reads value head g % Gv)
+        const bf16* vbase = v_pages + ((size_t)(page < 0 ? 0 : page) * Gv + g % Gv) * HD * ps + (size_t)blk * ND * 512 + lane * 8;
         bf16x8 kf[2][NC];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
@@ -241,8 +242,12 @@ extern "C" size_t spite_attn_decode_workspace(int T, int H, int hd, int n_splits
 extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* out, void* workspace,
                                  const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
-                                 float scale, float softcap, const float* slopes, int n_splits, hipStream_t st) {
+                                 float scale, float softcap, const float* slopes, int n_splits, int value_heads,
+                                 hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_decode: scale %g, score cap %g", scale, softcap);
+    // value pages [pages][value_heads][hd][page]: kv head g reads value head g % value_heads (0: as many as kv heads)
+    if (value_heads <= 0) value_heads = G;
+    SP_REQUIRE(G % value_heads == 0, "attn_decode: %d key heads over %d value heads", G, value_heads);
     SP_REQUIRE(T >= 0 && H > 0 && G > 0 && H % G == 0, "attn_decode: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(H / G <= 16, "attn_decode: %d query heads per kv head, at most 16", H / G);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_decode: head size %d (this kernel has 64 and 128)", hd);
@@ -256,13 +261,13 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
     if (hd == 128) {
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
@@ -308,5 +313,5 @@ extern "C" int spite_attn_decode_static(const void* q, const void* k_pages, cons
     SP_REQUIRE(e == hipSuccess && ptr != nullptr, "attn_decode_static: no address for the scratch array: %s",
                hipGetErrorString(e));
     return spite_attn_decode(q, k_pages, v_pages, out, ptr, positions, seq_of_token, block_table, max_blocks, T, H, G,
-                             hd, page_size, vis, span, scale, 0.f, nullptr, n_splits, st);
+                             hd, page_size, vis, span, scale, 0.f, nullptr, n_splits, 0, st);
 }

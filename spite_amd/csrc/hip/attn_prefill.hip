@@ -56,7 +56,7 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                          const int* __restrict__ block_table, int max_blocks, int tile_q,
                          int H, int G, int ps, int vis, int span, float scale_log2e, float cap_ratio,
-                         const float* __restrict__ slopes, float inv_scale, int n_splits) {
+                         const float* __restrict__ slopes, float inv_scale, int n_splits, int Gv) {
     constexpr int NS = HD / 16;                      // steps of 16 head elements in the score product
     constexpr int NDT = HD / 32;                     // 32-row tiles of the output
     constexpr int NC = HD / 32;                      // chunks of a K tile row
@@ -137,7 +137,8 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         // a page that is absent is read as page 0: its keys are masked or poisoned below, its
         // values taken as zero
         pg = pg < 0 ? 0 : pg;
-        const size_t at = ((size_t)pg * G + g) * (size_t)ps * HD + (size_t)((key % ps) >> 5) * RUN + lane * 8;
+        // (value heads may be fewer than key heads: key head g reads value head g % Gv)
+        const size_t at = (is_v ? (size_t)pg * Gv + g % Gv : (size_t)pg * G + g) * (size_t)ps * HD + (size_t)((key % ps) >> 5) * RUN + lane * 8;
         const bf16* src = (is_v ? v_pages : k_pages) + at;
         bf16* dst = (is_v ? Vs : Ks) + buf * STEP + hx * RUN;
 #pragma unroll
@@ -422,7 +423,7 @@ template <int HD, bool EXTRA>
 static int launch_prefill(const void* q, const void* k_pages, const void* v_pages, void* out, float* part, const int* positions,
                           const int* cu_seqlens, int n_seqs, const int* block_table, int max_blocks, int tile_q,
                           long n_tiles, int H, int G, int page_size, int vis, int span, float sl, float cr,
-                          const float* slopes, float inv_scale, int n_splits, hipStream_t st) {
+                          const float* slopes, float inv_scale, int n_splits, int Gv, hipStream_t st) {
     const size_t sh = (size_t)2 * 2 * PF_KEYS * HD * sizeof(bf16);
     static bool allowed = false;          // one flag per instantiation: more LDS than the default limit
     if (!allowed) {
@@ -432,7 +433,7 @@ static int launch_prefill(const void* q, const void* k_pages, const void* v_page
     }
     attn_prefill_kernel<HD, EXTRA><<<dim3((unsigned)(n_tiles * G * n_splits)), 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages,
         (const bf16*)v_pages, (bf16*)out, part, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size,
-        vis, span, sl, cr, slopes, inv_scale, n_splits);
+        vis, span, sl, cr, slopes, inv_scale, n_splits, Gv);
     SP_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -473,8 +474,11 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
                                   const int* positions, const int* cu_seqlens, const int* counts, int n_seqs,
                                   const int* block_table, int max_blocks, int H, int G, int hd, int page_size,
                                   int vis, int span, float scale, float softcap, const float* slopes, int n_splits,
-                                  hipStream_t st) {
+                                  int value_heads, hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_prefill: scale %g, score cap %g", scale, softcap);
+    // value pages [pages][value_heads][hd][page]: kv head g reads value head g % value_heads (0: as many as kv heads)
+    if (value_heads <= 0) value_heads = G;
+    SP_REQUIRE(G % value_heads == 0, "attn_prefill: %d key heads over %d value heads", G, value_heads);
     SP_REQUIRE(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0, "attn_prefill: %d query heads over %d kv heads", H, G);
     SP_REQUIRE(H / G <= PF_COLS, "attn_prefill: %d query heads per kv head, at most %d", H / G, PF_COLS);
     SP_REQUIRE(hd == 64 || hd == 128, "attn_prefill: head size %d (this kernel has 64 and 128)", hd);
@@ -494,7 +498,7 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
     const float sl = scale * 1.4426950408889634f, cr = softcap > 0.f ? scale / softcap : 0.f;
     const bool extra = cr > 0.f || slopes != nullptr;
 #define SP_PF(HDV, EX) launch_prefill<HDV, EX>(q, k_pages, v_pages, out, (float*)workspace, positions, cu_seqlens, n_seqs, \
-        block_table, max_blocks, tile_q, tiles, H, G, page_size, vis, span, sl, cr, slopes, 1.0f / scale, n_splits, st)
+        block_table, max_blocks, tile_q, tiles, H, G, page_size, vis, span, sl, cr, slopes, 1.0f / scale, n_splits, value_heads, st)
     const int rc = hd == 128 ? (extra ? SP_PF(128, true) : SP_PF(128, false)) : (extra ? SP_PF(64, true) : SP_PF(64, false));
 #undef SP_PF
     if (rc != 0 || n_splits == 1) return rc;

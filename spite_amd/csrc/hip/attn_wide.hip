@@ -20,8 +20,10 @@
 // row).  x = row + bias; with `wq` / `wk` the q and the k region are each divided by the root mean
 // square of the whole region and multiplied by their weights; then the first `rot` elements
 // of every q and k head turn by pos * inv_freq[i] in pairs (i, i + rot/2); with `inv_freq_v` the
-// values turn by pos * inv_freq_v[m] in pairs (m, m + Vd/2).  Keys go to [page][GK][offset][D],
-// values to [page][GV][Vd][offset] (or the operand order of common.h).
+// values turn by pos * inv_freq_v[m] in pairs (m, m + Vd/2).  Keys go to [page][GK][offset][Dp],
+// values to [page][GV][Vd][offset] (or the operand order of common.h).  Dp >= D is the width that
+// queries and keys are stored with: the elements behind D are written as zeros (a head narrower than
+// what an attention kernel takes is widened this way; zeros add nothing to a score).
 template <typename T>
 __global__ __launch_bounds__(WIDE_NT)
 void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restrict__ bias,
@@ -29,7 +31,7 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
                         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                         const int* __restrict__ positions, const int* __restrict__ slot_map,
                         const float* __restrict__ inv_freq, int rot, const float* __restrict__ inv_freq_v,
-                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled) {
+                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp) {
     extern __shared__ float sm[];
     __shared__ float red[WIDE_NT / 64];
     const int rh = rot >> 1, vh = inv_freq_v ? (Vd >> 1) : 0;
@@ -74,11 +76,11 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
             return x;
         };
         T* dst = nullptr;
-        if (is_q) dst = q_out + ((size_t)t * HQ + hh) * D;
-        else dst = k_pages + (page * GK + (hh - HQ)) * (size_t)ps * D;
+        if (is_q) dst = q_out + ((size_t)t * HQ + hh) * Dp;
+        else dst = k_pages + (page * GK + (hh - HQ)) * (size_t)ps * Dp;
         auto store = [&](int c, float v) {
             if (is_q) dst[c] = from_f32<T>(v);
-            else dst[sp_k_index(off, c, D, k_tiled)] = from_f32<T>(v);
+            else dst[sp_k_index(off, c, Dp, k_tiled)] = from_f32<T>(v);
         };
         if (i < rh) {
             const float a = load(i), b = load(i + rh);
@@ -88,6 +90,11 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
             const int c = rot + (i - rh);
             store(c, load(c));
         }
+    }
+    for (int it = tid; it < (HQ + (slot >= 0 ? GK : 0)) * (Dp - D); it += WIDE_NT) {
+        const int hh = it / (Dp - D), c = D + it % (Dp - D);
+        if (hh < HQ) q_out[((size_t)t * HQ + hh) * Dp + c] = from_f32<T>(0.f);
+        else k_pages[(page * GK + (hh - HQ)) * (size_t)ps * Dp + sp_k_index(off, c, Dp, k_tiled)] = from_f32<T>(0.f);
     }
     if (slot < 0) return;
     const int vitems = Vd - vh;
@@ -111,14 +118,16 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
                                  float eps, void* q_out, void* k_pages, void* v_pages, const int* positions,
                                  const int* slot_map, const float* inv_freq, int rot, const float* inv_freq_v,
                                  int T, int HQ, int GK, int GV, int D, int Vd, int page_size, int k_tiled, int v_tiled,
-                                 hipStream_t st) {
+                                 int Dp, hipStream_t st) {
+    if (Dp <= 0) Dp = D;
+    SP_REQUIRE(Dp >= D, "qkv_prepare: heads of %d stored with %d elements", D, Dp);
     SP_REQUIRE(T >= 0 && HQ > 0 && GK > 0 && GV > 0 && D > 0 && Vd > 0 && page_size > 0, "qkv_prepare: bad sizes");
     SP_REQUIRE(ld >= (HQ + GK) * D + GV * Vd, "qkv_prepare: rows of %d elements for %d", ld, (HQ + GK) * D + GV * Vd);
     SP_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "qkv_prepare: %d turning elements of a head of %d", rot, D);
     SP_REQUIRE(rot == 0 || inv_freq, "qkv_prepare: rotation needs a frequency table");
     SP_REQUIRE(!inv_freq_v || Vd % 2 == 0, "qkv_prepare: values of %d elements cannot turn in pairs", Vd);
     SP_REQUIRE(!slot_map || (k_pages && v_pages), "qkv_prepare: writing the cache needs its pages");
-    SP_REQUIRE(!k_tiled || (dtype == SP_BF16 && D % 32 == 0 && page_size % 32 == 0), "qkv_prepare: keys of %d in operand order", D);
+    SP_REQUIRE(!k_tiled || (dtype == SP_BF16 && Dp % 32 == 0 && page_size % 32 == 0), "qkv_prepare: keys of %d in operand order", Dp);
     SP_REQUIRE(!v_tiled || (dtype == SP_BF16 && Vd % 32 == 0 && page_size % 32 == 0), "qkv_prepare: values of %d in operand order", Vd);
     SP_REQUIRE(eps > 0.f || (!wq && !wk), "qkv_prepare: the norm needs an eps");
     if (T == 0) return 0;
@@ -126,10 +135,10 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
     SP_REQUIRE(sh <= 48 * 1024, "qkv_prepare: heads too wide");
     if (dtype == SP_F32)
         qkv_prepare_kernel<float><<<T, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
-            (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled);
+            (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp);
     else if (dtype == SP_BF16)
         qkv_prepare_kernel<bf16><<<T, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled);
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp);
     else return sp_fail("qkv_prepare: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("qkv_prepare");
     return 0;

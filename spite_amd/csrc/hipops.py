@@ -48,11 +48,11 @@ def lib():
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_filter_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, I, P],
-            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P],
+            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, P, I, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, P, I, I, P],
             "spite_attn_prefill_splits": [P, I, I, I, L],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
@@ -63,7 +63,7 @@ def lib():
             "spite_router_topk": [P, P, P, P, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
-            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, P],
+            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, I, P],
             "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
             "spite_attn_finish": [P, I, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
             "spite_token_shift": [P, P, I, P, P, P, P, P, I, I, I, P],
@@ -111,9 +111,9 @@ def _ptr_rows(t, name):
     return _ptr(t, name)
 
 
-def _check_pages(k_pages, v_pages, G, page_size, hd, what):
-    """Key pages [n, G, page_size, hd]; value pages transposed, [n, G, hd, page_size]."""
-    if (tuple(k_pages.shape[1:]) != (G, page_size, hd) or tuple(v_pages.shape[1:]) != (G, hd, page_size)
+def _check_pages(k_pages, v_pages, G, page_size, hd, what, value_heads=None):
+    """Key pages [n, G, page_size, hd]; value pages transposed, [n, G (or value_heads), hd, page_size]."""
+    if (tuple(k_pages.shape[1:]) != (G, page_size, hd) or tuple(v_pages.shape[1:]) != (value_heads or G, hd, page_size)
             or k_pages.shape[0] != v_pages.shape[0]):
         raise KernelError(f"{what}: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
                           f"G={G} page={page_size} hd={hd}")
@@ -427,14 +427,16 @@ def attn_decode_workspace(T, H, hd, n_splits) -> int:
 
 
 def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
-                page_size, vis, span, scale, n_splits, softcap=0.0, slopes=None):
+                page_size, vis, span, scale, n_splits, softcap=0.0, slopes=None, value_heads=None):
     """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
-    keys, in operand order): every row of q is one query against its request's cache."""
+    keys, in operand order): every row of q is one query against its request's cache.
+    ``value_heads``: the value pages hold fewer heads than the key pages (kv head g reads value
+    head g % value_heads)."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_decode: bfloat16 only, got {q.dtype}")
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attn_decode: q or out too small")
-    _check_pages(k_pages, v_pages, G, page_size, hd, "attn_decode")
+    _check_pages(k_pages, v_pages, G, page_size, hd, "attn_decode", value_heads)
     if block_table.dim() != 2 or positions.numel() < T or seq_of_token.numel() < T:
         raise KernelError("attn_decode: metadata too small")
     if workspace.numel() * workspace.element_size() < attn_decode_workspace(T, H, hd, n_splits):
@@ -445,7 +447,7 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _ptr(workspace, "workspace"), _ptr(positions, "positions", torch.int32),
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap),
-        _slopes(slopes, H), int(n_splits), _stream()), "attn_decode")
+        _slopes(slopes, H), int(n_splits), int(value_heads or 0), _stream()), "attn_decode")
 
 
 def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
@@ -538,7 +540,7 @@ def attn_prefill_workspace(counts, H, G, hd, n_splits) -> int:
 
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
-                 H, G, hd, page_size, vis, span, scale, n_splits=1, scratch=None, softcap=0.0, slopes=None):
+                 H, G, hd, page_size, vis, span, scale, n_splits=1, scratch=None, softcap=0.0, slopes=None, value_heads=None):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
     operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
@@ -554,7 +556,7 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
     T = int(counts.sum())
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
         raise KernelError("attn_prefill: q or out too small")
-    _check_pages(k_pages, v_pages, G, page_size, hd, "attn_prefill")
+    _check_pages(k_pages, v_pages, G, page_size, hd, "attn_prefill", value_heads)
     if block_table.dim() != 2 or block_table.shape[0] < n_seqs or positions.numel() < T:
         raise KernelError("attn_prefill: metadata too small")
     if cu_seqlens.numel() < n_seqs + 1:
@@ -569,7 +571,7 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
         _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
         counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
         H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap), _slopes(slopes, H), n_splits,
-        _stream()), "attn_prefill")
+        int(value_heads or 0), _stream()), "attn_prefill")
 
 
 def _slopes(slopes, H):
@@ -753,23 +755,25 @@ def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg,
 # -------------------------------------------------------------------------------------------- keys and values of unequal shape
 def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D, Vd, page_size, *, bias=None,
                 norm_q=None, norm_k=None, eps=0.0, inv_freq=None, rot=0, inv_freq_v=None, write_kv=True,
-                k_tiled=False, v_tiled=False):
+                k_tiled=False, v_tiled=False, stored_dim=None):
     """Between a fused projection and the cache (see attn_wide.hip).  qkv: rows that begin with
     [HQ*D | GK*D | GV*Vd] (further columns are left alone); ``bias`` fp32 over those; ``norm_q`` /
     ``norm_k`` (fp32 [HQ*D], [GK*D]): weights of an RMS norm over the whole q and the whole k part;
     ``inv_freq`` (fp32 [rot/2]): the first ``rot`` elements of every q and k head turn in pairs
     (i, i + rot/2); ``inv_freq_v`` (fp32 [Vd/2]): the values turn in pairs (m, m + Vd/2).  q_out
-    [T, HQ*D]; key pages [pages, GK, page_size, D]; value pages [pages, GV, Vd, page_size]."""
+    [T, HQ*Dp]; key pages [pages, GK, page_size, Dp]; value pages [pages, GV, Vd, page_size], with
+    Dp = ``stored_dim`` (default D): queries and keys are stored that wide, zeros behind their D."""
     T = qkv.shape[0]
+    Dp = int(stored_dim or D)
     n = (HQ + GK) * D + GV * Vd
     if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n:
         raise KernelError(f"qkv_prepare: rows {tuple(qkv.shape)} for HQ={HQ} GK={GK} GV={GV} D={D} Vd={Vd}")
-    if q_out.numel() < T * HQ * D or positions.numel() < T:
+    if q_out.numel() < T * HQ * Dp or positions.numel() < T or Dp < D:
         raise KernelError("qkv_prepare: q_out or positions too small")
     if write_kv:
         if slot_map is None or slot_map.numel() < T:
             raise KernelError("qkv_prepare: slot map too small")
-        if tuple(k_pages.shape[1:]) != (GK, page_size, D) or tuple(v_pages.shape[1:]) != (GV, Vd, page_size) \
+        if tuple(k_pages.shape[1:]) != (GK, page_size, Dp) or tuple(v_pages.shape[1:]) != (GV, Vd, page_size) \
                 or k_pages.shape[0] != v_pages.shape[0]:
             raise KernelError(f"qkv_prepare: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
                               f"GK={GK} GV={GV} page={page_size} D={D} Vd={Vd}")
@@ -786,7 +790,7 @@ def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D
         _ptr(q_out, "q_out", dt), _ptr(k_pages, "k_pages", dt, not write_kv), _ptr(v_pages, "v_pages", dt, not write_kv),
         _ptr(positions, "positions", torch.int32), _ptr(slot_map, "slot_map", torch.int32) if write_kv else None,
         _ptr(inv_freq, "inv_freq", torch.float32, True), int(rot), _ptr(inv_freq_v, "inv_freq_v", torch.float32, True),
-        T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), _stream()), "qkv_prepare")
+        T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), Dp, _stream()), "qkv_prepare")
 
 
 def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, HQ, GK, GV, D, Vd, page_size, vis, span,

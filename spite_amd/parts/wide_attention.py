@@ -65,6 +65,11 @@ class WideAttention(Mixer):
             if pe is not None and (not pe.fused or pe.kernel_args().get("adjacent")):
                 raise ValueError("wide_attention: the position encoding must be a rotation in halves")
         self.HQ, self.GK = self.H * self.maps, self.G * self.maps
+        # the MFMA kernels take keys and values of one width, 64 or 128: narrower keys (and queries) are stored
+        # that wide in a bfloat16 run, zeros behind their own elements
+        self.Dk = self.D
+        if env.dtype == torch.bfloat16 and self.Vd in (64, 128) and self.D < self.Vd and self.HQ // self.GK <= 16:
+            self.Dk = self.Vd
         self.n_qkv = (self.HQ + self.GK) * self.D + self.G * self.Vd
         self.w_in = self.wo = self.b_in = self.w_qnorm = self.w_knorm = None
         self.inv_freq = self.inv_freq_v = None
@@ -134,22 +139,23 @@ class WideAttention(Mixer):
         if self.env.dtype == torch.bfloat16:
             if not self._mfma(page_size):
                 notes.append(f"attention runs on plain FMAs: keys of {self.D} and values of {self.Vd} elements, pages of "
-                             f"{page_size} (the MFMA kernels take equal widths of 64 or 128 and pages in multiples of 32)")
+                             f"{page_size} (the MFMA kernels take values of 64 or 128 with keys no wider, at most 16 query heads "
+                             f"a kv head, and pages in multiples of 32)")
             for name, w in (("q/k/v projection", self.w_in), ("output projection", self.wo)):
                 if w is not None:
                     notes += w.slow_reason(name)
         return notes
 
     def cache_need(self):
-        return CacheNeed(kv=KVNeed(self.GK, self.D, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G))
+        return CacheNeed(kv=KVNeed(self.GK, self.Dk, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G))
 
     def _mfma(self, page_size):
-        return (self.env.dtype == torch.bfloat16 and self.D == self.Vd and self.D in (64, 128) and page_size % 32 == 0
-                and self.HQ // self.GK <= 16 and self.maps == 1)
+        return (self.env.dtype == torch.bfloat16 and self.Dk == self.Vd and self.Vd in (64, 128) and page_size % 32 == 0
+                and self.HQ // self.GK <= 16)
 
     # ------------------------------------------------------------------ the step
     def _decode(self, q, o, ctx, cache, T):
-        HQ, GK, D = self.HQ, self.GK, self.D
+        HQ, GK, D = self.HQ, self.GK, self.Dk
         longest = cache.block_table.shape[1] * cache.page_size
         if self.visibility != "full":
             longest = min(longest, self.span + 32)
@@ -158,10 +164,10 @@ class WideAttention(Mixer):
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, HQ, D, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, HQ, GK, D, cache.page_size, self.visibility, self.span,
-                           self.scale, n_splits)
+                           self.scale, n_splits, value_heads=self.G)
 
     def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
-        HQ, GK, D = self.HQ, self.GK, self.D
+        HQ, GK, D = self.HQ, self.GK, self.Dk
         counts, starts = ctx.host.counts[lead:], ctx.host.starts[lead:]
         longest = int((starts + counts).max())
         if self.visibility != "full":
@@ -172,18 +178,18 @@ class WideAttention(Mixer):
             scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, HQ, GK, D, n_splits) // 4,), torch.float32)
         hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
                             cache.block_table[lead:], HQ, GK, D, cache.page_size, self.visibility, self.span, self.scale,
-                            n_splits=n_splits, scratch=scratch)
+                            n_splits=n_splits, scratch=scratch, value_heads=self.G)
 
     def forward(self, x, ctx, cache):
         T, ws = x.shape[0], ctx.ws
-        H, G, HQ, GK, D, Vd = self.H, self.G, self.HQ, self.GK, self.D, self.Vd
+        H, G, HQ, GK, D, Vd, Dk = self.H, self.G, self.HQ, self.GK, self.D, self.Vd, self.Dk
         proj = ws.take((T, self.n_in), x.dtype)
         linear(x, self.w_in, proj, ws=ws)
-        q = ws.take((T, HQ * D), x.dtype)
+        q = ws.take((T, HQ * Dk), x.dtype)
         hipops.qkv_prepare(proj, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, HQ, GK, G, D, Vd,
                            cache.page_size, bias=self.b_in, norm_q=self.w_qnorm, norm_k=self.w_knorm, eps=self.eps,
                            inv_freq=self.inv_freq, rot=self.rot, inv_freq_v=self.inv_freq_v, write_kv=cache.write,
-                           k_tiled=cache.tiled, v_tiled=cache.tiled)
+                           k_tiled=cache.tiled, v_tiled=cache.tiled, stored_dim=Dk)
         if cache.tiled and self._mfma(cache.page_size):
             a = ws.take((T, HQ * Vd), x.dtype)
             cu_tail, lead = ctx.derived[TAIL]
@@ -197,7 +203,7 @@ class WideAttention(Mixer):
             # two maps meet in a difference: keep them in fp32 until then
             a = ws.take((T, HQ * Vd), torch.float32 if self.maps == 2 else x.dtype)
             hipops.attn_wide(q, cache.k_pages, cache.v_pages, a, ctx.positions, ctx.seq_of_token, cache.block_table,
-                             T, HQ, GK, G, D, Vd, cache.page_size, self.visibility, self.span, self.scale,
+                             T, HQ, GK, G, Dk, Vd, cache.page_size, self.visibility, self.span, self.scale,
                              k_tiled=cache.tiled, v_tiled=cache.tiled)
         if self.maps == 2 or self.inv_freq_v is not None or self.head_gate:
             o = ws.take((T, H * Vd), x.dtype)

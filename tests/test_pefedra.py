@@ -330,6 +330,79 @@ def test_projection_to_cache_kernel(dtype, HQ, GK, GV, D, Vd, rot, ps, norm, tur
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,ps", [("float32", 8), ("bfloat16", 32)])
+def test_keys_stored_wider_than_they_are(dtype, ps):
+    """Queries and keys of 32 elements stored 64 wide: their own elements first, zeros behind them, also where
+    the page held something else before."""
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(5)
+    dt = getattr(torch, dtype)
+    T, HQ, GK, GV, D, Vd, Dp = 6, 4, 2, 1, 32, 64, 64
+    n = (HQ + GK) * D + GV * Vd
+    row = torch.randn(T, n, generator=g).to(dt)
+    positions = torch.arange(T, dtype=torch.int32)
+    slots = torch.tensor([ps + 3, ps + 4, 0, 1, 2 * ps - 1, 2 * ps], dtype=torch.int32)
+    tiled = dtype == "bfloat16"
+    kp = torch.full((3, GK, ps, Dp), float("nan"), dtype=dt, device="cuda:0")
+    vp = torch.zeros(3, GV, Vd, ps, dtype=dt, device="cuda:0")
+    q_out = torch.full((T, HQ * Dp), float("nan"), dtype=dt, device="cuda:0")
+    hipops.qkv_prepare(row.cuda(), q_out, kp, vp, positions.cuda(), slots.cuda(), HQ, GK, GV, D, Vd, ps, k_tiled=tiled, v_tiled=tiled,
+                       stored_dim=Dp)
+    want_q = torch.zeros(T, HQ, Dp, dtype=dt)
+    want_q[:, :, :D] = row[:, :HQ * D].view(T, HQ, D)
+    assert torch.equal(q_out.cpu().view(T, HQ, Dp), want_q)
+    want_k = torch.full((3, GK, ps, Dp), float("nan"), dtype=dt)
+    for t in range(T):
+        sl = int(slots[t])
+        want_k[sl // ps, :, sl % ps, :D] = row[t, HQ * D:(HQ + GK) * D].view(GK, D)
+        want_k[sl // ps, :, sl % ps, D:] = 0
+    if tiled:
+        want_k, _ = hipops.kv_operand_order(want_k.cuda(), vp)
+    assert torch.equal(torch.nan_to_num(kp.cpu(), nan=-7.0), torch.nan_to_num(want_k.cpu(), nan=-7.0))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hd,HQ,GK,GV", [(64, 8, 4, 2), (128, 4, 2, 1), (64, 2, 2, 2)])
+def test_matrix_unit_kernels_with_fewer_value_heads(hd, HQ, GK, GV):
+    """The prefill and decode kernels of the matrix units with value heads shared by several key heads, against
+    the plain kernel on the same pages: portions, and single tokens far into their requests."""
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(hd + GV)
+    ps, dev = 32, "cuda:0"
+    starts, lens = [70, 0, 23], [40, 17, 100]
+    totals = [s + c for s, c in zip(starts, lens)]
+    n_pages = sum(-(-t // ps) for t in totals) + 2
+    order = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((3, 8), -1, dtype=torch.int32)
+    for i, t in enumerate(totals):
+        for b in range(-(-t // ps)):
+            table[i, b] = order.pop()
+    kp, vp = hipops.kv_operand_order(torch.randn(n_pages, GK, ps, hd, generator=g).bfloat16().to(dev),
+                                     torch.randn(n_pages, GV, hd, ps, generator=g).bfloat16().to(dev))
+    scale = 1.0 / math.sqrt(hd)
+    for decode in (False, True):
+        ln = [1, 1, 1] if decode else lens
+        st = [t - 1 for t in totals] if decode else starts
+        T = sum(ln)
+        q = (torch.randn(T, HQ * hd, generator=g) * 1.5).bfloat16().to(dev)
+        positions = torch.tensor([s + j for s, c in zip(st, ln) for j in range(c)], dtype=torch.int32, device=dev)
+        seq = torch.tensor([i for i, c in enumerate(ln) for _ in range(c)], dtype=torch.int32, device=dev)
+        cu = torch.tensor(np.concatenate([[0], np.cumsum(ln)]), dtype=torch.int32, device=dev)
+        ref = torch.empty(T, HQ * hd, device=dev)
+        hipops.attn_wide(q, kp, vp, ref, positions, seq, table.to(dev), T, HQ, GK, GV, hd, hd, ps, "window", 90, scale, k_tiled=True, v_tiled=True)
+        out = torch.full((T, HQ * hd), float("nan"), dtype=torch.bfloat16, device=dev)
+        if decode:
+            n_splits = 2
+            scratch = torch.empty(hipops.attn_decode_workspace(T, HQ, hd, n_splits) // 4, device=dev)
+            hipops.attn_decode(q, kp, vp, out, scratch, positions, seq, table.to(dev), T, HQ, GK, hd, ps, "window", 90, scale, n_splits,
+                               value_heads=GV)
+        else:
+            hipops.attn_prefill(q, kp, vp, out, positions, cu, np.asarray(ln), table.to(dev), HQ, GK, hd, ps, "window", 90, scale,
+                                value_heads=GV)
+        assert float((out.float() - ref).abs().max()) < 0.02 * float(ref.abs().max())
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H_,Vd", [(3, 14), (4, 64), (1, 130)])
 def test_attention_finish_kernel(dtype, H_, Vd):
