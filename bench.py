@@ -168,7 +168,8 @@ class KernelTimes:
     NAMES = ("embed", "add_rmsnorm", "rope_kvwrite", "router_top1", "moe_plan", "convert", "gemm_generic",
              "attn_generic", "gemm_skinny", "gemm_mfma", "gemm_tiled", "attn_decode", "attn_prefill",
              "sample_rows", "argmax_rows", "filter_rows", "latent_prepare", "attn_latent_generic", "attn_latent_mfma",
-             "router_topk", "moe_combine", "gated_rows", "add_into")
+             "router_topk", "moe_combine", "gated_rows", "add_into",
+             "qkv_prepare", "attn_wide", "attn_finish", "token_shift", "act_rows")
 
     def __init__(self):
         import torch
@@ -217,13 +218,38 @@ class KernelTimes:
 # first one's cache.  Llama 4 at the same width, heads (head size 128, a kv head for every four),
 # experts and layers, its one routed and one shared expert as wide as the Ravenex token's experts
 # together, its rotating layers reading a window of the same length.
+# ``--design pefedra``: the Pefedra design beside Llama 4 with dense layers only.  Pefedra: three layers of
+# ``attention_2`` (heads of 128, the first 64 elements turning, a kv head for every four) to one of ``attention``
+# (half as many heads, two score maps of 64 each over values of 128: the same score and value products a
+# token as the other layers), a window of 4,096 everywhere, an ungated feed-forward 1.5 times as wide as
+# Llama 4's gated one (``dense_ff``), so that both have the same products a token.
 DESIGN_SIZES = {
-    "2k": dict(width=2048, heads=16, experts=16, top=4, expert_ff=1024, shared_ff=2048),
-    "5k": dict(width=5120, heads=40, experts=16, top=2, expert_ff=4096, shared_ff=8192),
+    "2k": dict(width=2048, heads=16, experts=16, top=4, expert_ff=1024, shared_ff=2048, dense_ff=8192),
+    "5k": dict(width=5120, heads=40, experts=16, top=2, expert_ff=4096, shared_ff=8192, dense_ff=16384),
 }
 
 
-def design_configs(sz, layers, window, vocab):
+def pefedra_configs(sz, layers, window, vocab):
+    H = sz["heads"]
+    gated = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
+             "rot": {"base": 500000.0, "dims": 64}}
+    two_maps = {"heads": H // 2, "kv_heads": max(1, H // 8), "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.5,
+                "mask": {"size": window}, "rot": {"base": 50000.0, "dims": 64, "scaling": {"factor": 8.0}}}
+    mlp = {"kind": "dense", "ff": sz["dense_ff"] * 3 // 2}
+    pefedra = {"architecture": "Pefedra", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
+               "torch_dtype": "bfloat16",
+               "layers": [{"type": "attention", "mixer": two_maps, "mlp": mlp} if i % 4 == 2 else
+                          {"type": "attention_2", "mixer": gated, "mlp": mlp} for i in range(layers)]}
+    llama = dict(SCOUT, num_hidden_layers=layers, hidden_size=sz["width"], num_attention_heads=H,
+                 num_key_value_heads=max(1, H // 4), head_dim=128, num_local_experts=0, moe_layers=[], interleave_moe_layer_step=0,
+                 intermediate_size=sz["dense_ff"], intermediate_size_mlp=sz["dense_ff"], vocab_size=vocab,
+                 attention_chunk_size=window, no_rope_layers=None, rope_scaling=None, attention_local_kind="window")
+    return {"pefedra": pefedra, "llama4": llama}
+
+
+def design_configs(sz, layers, window, vocab, design="ravenex"):
+    if design == "pefedra":
+        return pefedra_configs(sz, layers, window, vocab)
     mix = lambda kv_from: dict({"heads": sz["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
                                 "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5},
                                **({} if kv_from is None else {"kv_from": kv_from}))
@@ -252,7 +278,7 @@ def design_comparison(args):
     page, V, layers, window = 64, 32768, args.layers or 4, 4096
     batch, context, T = args.batch, args.context, args.prefill_tokens
     rng = np.random.RandomState(0)
-    out = {"metric": "prefill and decode tok/s of the Ravenex design beside Llama 4 at equal sizes (random weights)",
+    out = {"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside Llama 4 at equal sizes (random weights)",
            "value": None, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
            "higher_is_better": True, "data": "synthetic: random weights, uniform-random token ids, context pages filled with random values",
            "config": {"layers": layers, "window": window, "global_batch": batch, "seq_len": context, "prefill_tokens": T, "vocab": V},
@@ -260,7 +286,7 @@ def design_comparison(args):
     for name in [x for x in args.design_sizes.split(",") if x.strip()]:
         sz = DESIGN_SIZES[name]
         out["sizes"][name] = {"size": sz}
-        for design, cfg in design_configs(sz, layers, window, V).items():
+        for design, cfg in design_configs(sz, layers, window, V, args.design).items():
             per_req = -(-(context + args.runs * args.steps + args.warmup + 16) // page) * page
             eng = Engine(cfg, dtype=args.dtype, page_size=page, cache_tokens=max(batch * per_req, T + 2 * page),
                          max_requests=batch, max_batch_tokens=max(T, batch), random_weights=True, seed=0,
@@ -578,8 +604,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--runs", type=int, default=3, help="how many times the K steps are timed")
     ap.add_argument("--workload", default="decode", choices=["decode", "longctx", "serve", "designs"],
-                    help="designs: the Ravenex design beside Llama 4 at equal sizes (see DESIGN_SIZES)")
+                    help="designs: another design (--design) beside Llama 4 at equal sizes (see DESIGN_SIZES)")
     ap.add_argument("--design-sizes", default="2k,5k", help="designs: which of DESIGN_SIZES, comma separated")
+    ap.add_argument("--design", default="ravenex", choices=["ravenex", "pefedra"],
+                    help="designs: which design runs beside Llama 4 (pefedra: against Llama 4 with dense layers only)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (memory or time)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)

@@ -141,6 +141,16 @@ __device__ __forceinline__ float sp_gate_act(float g, int act, bool fast) {
     return g / (1.0f + (fast ? __expf(-g) : expf(-g)));
 }
 
+// An activation on its own (no gate): SP_UNARY_GELU 0.5 z (1 + erf(z / sqrt 2)), SP_UNARY_GELU_TANH,
+// SP_UNARY_SILU; fp32, the accurate routines.  The product kernels take one as the epilogue of a plain
+// product: their `glu` argument carries it in the bits above the gate's code (glu = unary << 4).
+enum { SP_UNARY_GELU = 1, SP_UNARY_GELU_TANH = 2, SP_UNARY_SILU = 3 };
+__device__ __forceinline__ float sp_unary(float z, int act) {
+    if (act == SP_UNARY_GELU) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (act == SP_UNARY_GELU_TANH) return sp_gate_act(z, SP_ACT_GELU_TANH, false);
+    return sp_gate_act(z, SP_ACT_SILU, false);
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<bf16>(bf16 v) { return (float)v; }

@@ -82,6 +82,8 @@ __device__ __forceinline__ float wave_dot_row(const float* __restrict__ w, const
 // v += mult * dn[r] * 1/sqrt(mean(dn[r]^2) + eps_n) * wn  (a sublayer's result that passes a norm
 // of its own and a constant before it joins the residual stream).  With `plain_out`, out[i] is v
 // itself in the output's dtype (no norm, `w` unused): the stream as a later product's operand.
+// With `w2` and `out2` the row goes out a second time, normed with the weights w2 (two norms of
+// one stream: a layer whose mixer and feed-forward read the same rows), in `out`'s dtype.
 #define NORM_NT 512
 #define NORM_MAX_V 8     // widths up to 4*NT*MAX_V = 16384 stay in registers
 template <typename TO, bool VEC>
@@ -92,7 +94,7 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                         const int* __restrict__ rows, int d, float eps, int write_h,
                         const float* __restrict__ proj, float* __restrict__ proj_out, int P,
                         const float* __restrict__ dn, const float* __restrict__ wn, float mult, float eps_n,
-                        int plain_out) {
+                        int plain_out, const float* __restrict__ w2, TO* __restrict__ out2) {
     __shared__ float red[NORM_NT / 64];
     extern __shared__ __attribute__((aligned(16))) float ys[];            // [d] if proj
     const int i = blockIdx.x;
@@ -137,7 +139,7 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                 ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
             }
         }
-        if (!out && !out32 && !proj) return;               // the additions were all that was asked for
+        if (!out && !out32 && !proj && !out2) return;      // the additions were all that was asked for
         const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
         const float scale = 1.0f / sqrtf(ms + eps);
 #pragma unroll
@@ -152,15 +154,23 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
                 }
                 if (out32) ((f32x4*)(out32 + (size_t)i * d))[c] = y;
                 if (proj) ((f32x4*)ys)[c] = y;
-                if (out) {
+                auto put = [&](TO* dst, const f32x4& yy) {
                     if constexpr (sizeof(TO) == 2) {             // four bf16 in one 8-byte store (d % 4 == 0 here)
                         bf16x4 o4;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) o4[e] = (bf16)y[e];
-                        *(bf16x4*)((bf16*)out + (size_t)i * d + 4 * c) = o4;
+                        for (int e = 0; e < 4; ++e) o4[e] = (bf16)yy[e];
+                        *(bf16x4*)((bf16*)dst + (size_t)i * d + 4 * c) = o4;
                     } else {
-                        ((f32x4*)((float*)out + (size_t)i * d))[c] = y;
+                        ((f32x4*)((float*)dst + (size_t)i * d))[c] = yy;
                     }
+                };
+                if (out) put(out, y);
+                if (out2) {                                      // the same row under a second norm's weights
+                    const f32x4 ww = ((const f32x4*)w2)[c];
+                    f32x4 y2;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y2[e] = v[u][e] * scale * ww[e];
+                    put(out2, y2);
                 }
             }
         }
@@ -179,7 +189,7 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
             if (write_h) hr[c] = x;
             ss += x * x;
         }
-        if (!out && !out32 && !proj) return;
+        if (!out && !out32 && !proj && !out2) return;
         const float ms = block_sum<NORM_NT>(ss, red) / (float)d;
         const float scale = 1.0f / sqrtf(ms + eps);
         for (int c = threadIdx.x; c < d; c += NORM_NT) {
@@ -187,6 +197,7 @@ void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ d1,
             if (!write_h) { if (a) x += a[c]; if (b) x += b[c]; if (nr) x += nr[c] * sn * wn[c]; }
             const float y = plain_out ? x : x * scale * w[c];
             if (out) out[(size_t)i * d + c] = from_f32<TO>(y);
+            if (out2) out2[(size_t)i * d + c] = from_f32<TO>(x * scale * w2[c]);
             if (out32) out32[(size_t)i * d + c] = y;
             if (proj) ys[c] = y;
         }
@@ -206,7 +217,8 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
                                  int out_dtype, float* out32, const int* rows, int n_rows, int d,
                                  float eps, int write_h, const float* proj, float* proj_out, int P,
                                  const float* dn, const float* wn, float mult, float eps_n, int plain_out,
-                                 hipStream_t st) {
+                                 const float* w2, void* out2, hipStream_t st) {
+    SP_REQUIRE(!out2 || w2, "add_rmsnorm: a second output needs the second norm's weight");
     SP_REQUIRE(n_rows >= 0 && d > 0 && eps > 0.f, "add_rmsnorm: bad sizes rows=%d d=%d eps=%g", n_rows, d, eps);
     SP_REQUIRE(!dn || (wn && eps_n > 0.f), "add_rmsnorm: a normed increment needs its weight and eps");
     SP_REQUIRE(w || plain_out || (!out && !out32 && !proj), "add_rmsnorm: a normed output needs the norm's weight");
@@ -215,9 +227,10 @@ extern "C" int spite_add_rmsnorm(float* h, const float* d1, const float* d2, con
     SP_REQUIRE(sh <= 48 * 1024, "add_rmsnorm: rows of %d do not fit the projection's LDS", d);
     if (n_rows == 0) return 0;
     auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
-    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32) && al(out) && al(dn) && al(wn);
-#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out); \
-        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out); } while (0)
+    const bool vec = d % 4 == 0 && d <= 4 * NORM_NT * NORM_MAX_V && al(h) && al(d1) && al(d2) && al(w) && al(out32) && al(out) && al(dn) && al(wn)
+        && al(w2) && al(out2);
+#define SP_NORM(TO) do { if (vec) add_rmsnorm_kernel<TO, true><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out, w2, (TO*)out2); \
+        else add_rmsnorm_kernel<TO, false><<<n_rows, NORM_NT, sh, st>>>(h, d1, d2, w, (TO*)out, out32, rows, d, eps, write_h, proj, proj_out, P, dn, wn, mult, eps_n, plain_out, w2, (TO*)out2); } while (0)
     if (out_dtype == SP_F32) SP_NORM(float);
     else if (out_dtype == SP_BF16) SP_NORM(bf16);
     else return sp_fail("add_rmsnorm: unknown dtype %d", out_dtype);

@@ -157,10 +157,15 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
         }
         if (a_scale) { const float sc = a_scale[s]; v *= sc; u *= sc; }
         if (GLU) v = sp_gate_act(v, act, true) * u;
+        else if (act < 0) v = sp_unary(v, -act);                 // a plain product with an activation of its own
         const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
         Y[yr * ldy + n] = from_f32<TY>(v);
     }
 }
+
+// The activation of the product that the calling thread is launching: the gate's code, or minus the
+// code of a plain product's own activation (set by the entry point).
+static thread_local int g_skinny_act = 0;
 
 template <int R, int G, int S, int NW>
 static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* Y, int y_dtype, int ldy, int M, int N,
@@ -181,7 +186,7 @@ static int launch_skinny(const void* X, int ldx, const void* W, long wgs, void* 
         if (sh > 48 * 1024) { hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh); \
             if (e != hipSuccess) return sp_fail("gemm_skinny: cannot get %zu bytes of LDS: %s", sh, hipGetErrorString(e)); } \
         kern<<<grid, NW * 64, sh, st>>>((const bf16*)X, ldx, (const bf16*)W, wgs, (TY*)Y, ldy, M, N, K, offsets, \
-                                        n_groups, a_rows, a_scale, y_rows, glu); } while (0)
+                                        n_groups, a_rows, a_scale, y_rows, g_skinny_act); } while (0)
     if (glu) { if (y_dtype == SP_BF16) SP_SK(true, bf16); else SP_SK(true, float); }
     else { if (y_dtype == SP_BF16) SP_SK(false, bf16); else SP_SK(false, float); }
 #undef SP_SK
@@ -197,6 +202,10 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
                                  const float* a_scale, const int* y_rows, int glu, int max_rows, int variant,
                                  int w_tiled, int live_groups, hipStream_t st) {
     SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+    const int unary = glu >> 4;
+    glu &= 15;
+    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_SILU, "gemm_skinny: activation code %d", glu | (unary << 4));
+    g_skinny_act = glu ? glu : -unary;
     SP_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, ldx);
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_skinny: output dtype %d", y_dtype);

@@ -277,6 +277,10 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
                 float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) v[i] = acc[a][b][i] * sc;
+                if (act < 0) {                                   // a plain product with an activation of its own
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = sp_unary(v[i], -act);
+                }
                 put4(yrow, ncol[a] + q * 4, v);
             }
         }
@@ -364,6 +368,7 @@ extern "C" int spite_gemm_tiled_split(const void* X, int ldx, const void* W, voi
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     const int nu = K / 64;
     SP_REQUIRE(k_splits >= 2 && workspace, "gemm_tiled: a split call needs at least two runs and a workspace");
+    g_gate_act = SP_ACT_SILU;                        // partial sums take no activation, whatever the thread's last call had
     SP_REQUIRE(((nu + k_splits - 1) / k_splits) * (k_splits - 1) < nu, "gemm_tiled: %d runs over %d steps leave a run empty", k_splits, nu);
     const size_t stride = (size_t)M * N;
     int rc = launch_tiled_kernel<8, 1, 8, false, float, true>(X, ldx, W, 0, workspace, N, M, N, K, nullptr, 1, nullptr, nullptr, nullptr,
@@ -393,7 +398,10 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(y_dtype == SP_BF16 || y_dtype == SP_F32, "gemm_tiled: output dtype %d", y_dtype);
     SP_REQUIRE(!offsets || n_groups > 0, "gemm_tiled: grouped call without groups");
     SP_REQUIRE(shape >= 0 && shape <= 6, "gemm_tiled: tile shape %d", shape);
-    g_gate_act = glu ? glu : SP_ACT_SILU;
+    const int unary = glu >> 4;
+    glu &= 15;
+    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_SILU, "gemm_tiled: activation code %d", glu | (unary << 4));
+    g_gate_act = glu ? glu : (unary ? -unary : SP_ACT_SILU);
     if (M == 0) return 0;
     if (shape == 0) {
         // Tiles come in whole numbers per CU: a plain product whose 128-row tiles leave many of the

@@ -1,5 +1,4 @@
-// Small row-wise kernels: the token shift of a mixer's input, an activation applied in place,
-// and the two norms of a layer whose mixer and feed-forward read the same stream.
+// Small row-wise kernels: the token shift of a mixer's input and an activation applied in place.
 #include "common.h"
 
 // ------------------------------------------------------------------ token shift
@@ -45,14 +44,7 @@ extern "C" int spite_token_shift(const float* x, void* y, int y_dtype, const flo
 }
 
 // ------------------------------------------------------------------ activation in place
-// SP_UNARY_GELU: 0.5 z (1 + erf(z / sqrt 2)); SP_UNARY_GELU_TANH; SP_UNARY_SILU.  fp32 inside.
-enum { SP_UNARY_GELU = 1, SP_UNARY_GELU_TANH = 2, SP_UNARY_SILU = 3 };
-__device__ __forceinline__ float sp_unary(float z, int act) {
-    if (act == SP_UNARY_GELU) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
-    if (act == SP_UNARY_GELU_TANH) return sp_gate_act(z, SP_ACT_GELU_TANH, false);
-    return sp_gate_act(z, SP_ACT_SILU, false);
-}
-
+// (the activations: sp_unary in common.h)
 template <typename T>
 __global__ __launch_bounds__(256)
 void act_rows_kernel(T* __restrict__ x, size_t n, int act) {

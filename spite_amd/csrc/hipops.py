@@ -19,6 +19,9 @@ F32, BF16 = 0, 1
 VIS = build.visibility_codes()      # "full", "chunk", "window": name -> code
 # the gate's activation of a gated product act(gate) * up, as the kernels number them (True: silu)
 GATE_ACTS = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 2}
+# an activation of a plain product's own (no gate), as the kernels number them; the bf16 weight-stream and
+# tiled products take it in their epilogue, in the bits above the gate's code
+UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3}
 
 
 class KernelError(RuntimeError):
@@ -36,7 +39,7 @@ def lib():
         P, I, L, F = c_void_p, c_int, c_long, c_float
         sigs = {
             "spite_embed": [P, P, I, P, I, I, I, F, P],
-            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P, P, F, F, I, P],
+            "spite_add_rmsnorm": [P, P, P, P, P, I, P, P, I, I, F, I, P, P, I, P, P, F, F, I, P, P, P],
             "spite_rope_kvwrite": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, I, I, I, P, P, I, P],
             "spite_router_top1": [P, P, P, P, P, I, I, I, P],
             "spite_moe_plan": [P, P, P, P, P, P, P, I, I, I, I, P],
@@ -144,13 +147,14 @@ def add_rmsnorm_can_project(d: int) -> bool:
 
 
 def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True,
-                proj=None, proj_out=None, normed=None, plain_out=False):
+                proj=None, proj_out=None, normed=None, plain_out=False, w2=None, out2=None):
     """v = h[r] + d1[r] + d2[r] (stored back if write_h); out[i] = rmsnorm(v) * w with r =
     rows[i] or i.  h, d1, d2, out32 fp32; w fp32 [d]; out fp32 or bf16.  With ``proj`` ([P, d]
     fp32) also proj_out[i] = proj . (the normed row in fp32), [n, P] fp32: the same bits as
     ``router_top1`` gives for that row.  ``normed`` = (dn, wn, mult, eps_n): a further increment
     mult * rmsnorm(dn[r]; eps_n) * wn, normed on its way in.  ``plain_out``: out[i] = v itself (no
-    norm; ``w`` may be None).  With no output at all the call only adds."""
+    norm; ``w`` may be None).  ``w2`` / ``out2``: the same rows normed with a second weight (in the
+    dtype of ``out`` where there is one).  With no output at all the call only adds."""
     d = h.shape[-1]
     dn = wn = None
     mult = eps_n = 0.0
@@ -166,7 +170,9 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
             raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} does not match h {tuple(h.shape)}")
     if w is not None and w.numel() != d:
         raise KernelError(f"add_rmsnorm: weight of {w.numel()} for rows of {d}")
-    for name, t in (("out", out), ("out32", out32)):
+    if out2 is not None and (w2 is None or w2.numel() != d or (out is not None and out2.dtype != out.dtype)):
+        raise KernelError("add_rmsnorm: the second output needs a weight of its own and the first output's dtype")
+    for name, t in (("out", out), ("out32", out32), ("out2", out2)):
         if t is not None and (t.shape[-1] != d or t.shape[0] < n):
             raise KernelError(f"add_rmsnorm: {name} {tuple(t.shape)} is too small for {n} rows of {d}")
     if rows is None and n > h.shape[0]:
@@ -180,11 +186,13 @@ def add_rmsnorm(h, w, eps, out=None, out32=None, d1=None, d2=None, rows=None, n_
     _check(lib().spite_add_rmsnorm(
         _ptr(h, "h", torch.float32), _ptr(d1, "d1", torch.float32, True), _ptr(d2, "d2", torch.float32, True),
         _ptr(w, "w", torch.float32, True), _ptr(out, "out", None, True),
-        dtype_code(out.dtype) if out is not None else F32, _ptr(out32, "out32", torch.float32, True),
+        dtype_code(out.dtype) if out is not None else (dtype_code(out2.dtype) if out2 is not None else F32),
+        _ptr(out32, "out32", torch.float32, True),
         _ptr(rows, "rows", torch.int32, True), n, d, float(eps), int(write_h),
         _ptr(proj, "proj", torch.float32, True), _ptr(proj_out, "proj_out", torch.float32, True), P,
         _ptr(dn, "normed increment", torch.float32, True), _ptr(wn, "normed increment's weight", torch.float32, True),
-        float(mult), float(eps_n), int(bool(plain_out)), _stream()),
+        float(mult), float(eps_n), int(bool(plain_out)), _ptr(w2, "w2", torch.float32, True), _ptr(out2, "out2", None, True),
+        _stream()),
         "add_rmsnorm")
 
 
@@ -381,7 +389,7 @@ def _gemm_checks(a, w, y, M, N, K, offsets, n_groups, a_rows, a_scale, y_rows, g
 
 
 def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None,
-                glu=False, max_rows=None, variant=0, tiled=False, live_groups=0):
+                glu=False, max_rows=None, variant=0, tiled=False, live_groups=0, act=None):
     """Weight-streaming bf16 product for few rows (see gemm_skinny.hip); arguments as gemm_generic.
     ``max_rows``: the most rows a group can bring (default M).  ``tiled``: w is in MFMA operand
     order (``operand_order``).  ``live_groups``: a promise that at most this many groups hold rows
@@ -392,9 +400,18 @@ def gemm_skinny(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sc
     _check(lib().spite_gemm_skinny(
         _ptr_rows(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
-        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
+        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), _act_code(glu, act),
         int(max_rows if max_rows is not None else M), int(variant), int(bool(tiled)), int(live_groups), _stream()),
         "gemm_skinny")
+
+
+def _act_code(glu, act) -> int:
+    """The products' ``glu`` argument: the gate's code, or an activation of the product's own above it."""
+    if act is None:
+        return int(glu)
+    if glu or act not in UNARY_ACTS:
+        raise KernelError(f"product: activation {act!r} (known: {sorted(UNARY_ACTS)}; not beside a gate)")
+    return UNARY_ACTS[act] << 4
 
 
 def kv_tiled_ok(dtype, hd, page_size) -> bool:
@@ -500,7 +517,7 @@ def cu_count() -> int:
 
 
 def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
-               shape=0, part=None):
+               shape=0, part=None, act=None):
     """Tiled bf16 MFMA product for many rows over weights in operand order (``operand_order``;
     see gemm_tiled.hip); arguments as gemm_generic.  ``part`` (fp32 ``[runs, M, N]``, plain
     products only): the sum over k is cut into ``runs`` runs, each a workgroup of its own, whose
@@ -510,7 +527,7 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_tiled: bfloat16 operands only, got {a.dtype} and {w.dtype}")
     if part is not None:
-        if not (offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and shape == 0):
+        if not (offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and shape == 0 and act is None):
             raise KernelError("gemm_tiled: partial sums are for plain products only")
         if part.dim() != 3 or part.shape[1] != M or part.shape[2] != N or part.shape[0] < 2 or part.shape[0] > 32 \
                 or part.shape[0] * 2 > K // 64:
@@ -522,7 +539,7 @@ def gemm_tiled(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_sca
     _check(lib().spite_gemm_tiled(
         _ptr_rows(a, "a"), a.stride(0), _ptr(w, "w"), rows_w * K, _ptr_rows(y, "y"), dtype_code(y.dtype), y.stride(0),
         M, N, K, _ptr(offsets, "offsets", torch.int32, True), n_groups, _ptr(a_rows, "a_rows", torch.int32, True),
-        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), int(glu),
+        _ptr(a_scale, "a_scale", torch.float32, True), _ptr(y_rows, "y_rows", torch.int32, True), _act_code(glu, act),
         int(shape), _stream()), "gemm_tiled")
 
 
@@ -849,9 +866,6 @@ def token_shift(x, y, w, state, seq_of_token, cu_seqlens, seq_slots, keep=True):
         _ptr(state, "state", torch.float32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32), T, d, int(bool(keep)),
         _stream()), "token_shift")
-
-
-UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3}
 
 
 def act_rows(x, act):

@@ -201,23 +201,28 @@ class ParallelBlock(Block):
         h, ws = state["h"], ctx.ws
         T, d = h.shape
         d1, d2 = two_increments(h, state["pending"])
+        n2 = n2_32 = None
+        if self.ffn is not None:
+            n2 = ws.take((T, d), self.env.dtype)
+            if self.ffn.wants_f32_input:
+                n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
+        # both norms of the stream in one pass where the first norm's kernel can do that
+        paired = n2 is not None and n2_32 is None and getattr(self.norm1, "pairs_with", lambda o: False)(self.norm2)
+        both = {"second": (self.norm2, n2)} if paired else {}
         if self.shift is not None:
             # the shift blends fp32 rows; the mixer's input takes the run's dtype after it
             n32 = ws.take((T, d), torch.float32)
-            self.norm1.forward(h, None, d1=d1, d2=d2, out32=n32)
+            self.norm1.forward(h, None, d1=d1, d2=d2, out32=n32, **both)
             x = ws.take((T, d), self.env.dtype)
             self.shift.forward(n32, x, ctx, cache["shift"].state)        # a block with a shift has two caches, by name
         else:
             x = ws.take((T, d), self.env.dtype)
-            self.norm1.forward(h, x, d1=d1, d2=d2)
+            self.norm1.forward(h, x, d1=d1, d2=d2, **both)
         state["mixer_in"] = x
         if self.ffn is not None:
-            # the same stream (the increments are in it now) through the second norm
-            n2 = ws.take((T, d), self.env.dtype)
-            n2_32 = None
-            if self.ffn.wants_f32_input:
-                n2_32 = n2 if n2.dtype == torch.float32 else ws.take((T, d), torch.float32)
-            self.norm2.forward(h, n2, out32=None if n2_32 is n2 else n2_32, write_h=False)
+            if not paired:
+                # the same stream (the increments are in it now) through the second norm
+                self.norm2.forward(h, n2, out32=None if n2_32 is n2 else n2_32, write_h=False)
             state["ffn_in"] = (n2, n2_32)
 
     def _stage_mixer(self, state, ctx, cache):

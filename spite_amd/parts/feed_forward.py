@@ -89,8 +89,7 @@ class DenseMLP(FeedForward):
     def forward(self, x, x32, ctx, projected=None):
         T = x.shape[0]
         u = ctx.ws.take((T, self.F), x.dtype)
-        linear(x, self.w_up, u, ws=ctx.ws)
-        hipops.act_rows(u, self.activation)
+        linear(x, self.w_up, u, ws=ctx.ws, act=self.activation)
         y = ctx.ws.take((T, self.d), torch.float32)
         linear(u, self.w_down, y, ws=ctx.ws)
         return (y,)

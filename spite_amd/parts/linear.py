@@ -104,7 +104,7 @@ def grouped_tile_shape(tokens: int, groups: int, whole_groups: int = 0, col_tile
 
 
 def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, rows=None,
-           max_rows=None, tile_shape=0, live_groups=0, ws=None):
+           max_rows=None, tile_shape=0, live_groups=0, ws=None, act=None):
     """y[r] = W . x[r] for ``rows`` rows (default: all of x; for a row list: its length).
 
     With ``glu`` the weight holds gate rows then up rows and y = act(gate) * up: ``True`` or
@@ -112,7 +112,10 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
     ``max_rows``: the most rows that one group can bring (default: ``rows``).
     ``tile_shape``: the prefill product's tile (``grouped_tile_shape``), 0 = the library's choice.
     ``live_groups``: a promise that at most this many groups hold rows (0: none).
-    ``ws``: the workspace that temporaries (partial sums, widened rows) are taken from."""
+    ``ws``: the workspace that temporaries (partial sums, widened rows) are taken from.
+    ``act``: an activation on a plain product's result (``gelu``, ``gelu_tanh``, ``silu``; not beside
+    ``glu``): in the epilogue of the bfloat16 weight-stream and tiled products, a pass of its own after
+    the others."""
     tiled = False
     if isinstance(w, Weight):
         w, tiled = w.data, w.tiled
@@ -128,16 +131,19 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
         if most <= SKINNY_MAX_ROWS and not (tiled and most > 32 and offsets is None and N >= 65536):
             hipops.gemm_skinny(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                a_scale=a_scale, y_rows=y_rows, glu=glu, max_rows=most, tiled=tiled,
-                               live_groups=live_groups)
-        elif tiled:
-            plain = offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and tile_shape == 0
+                               live_groups=live_groups, act=act)
+            return
+        if tiled:
+            plain = offsets is None and a_rows is None and a_scale is None and y_rows is None and not glu and tile_shape == 0 \
+                and act is None
             runs = hipops.tiled_k_runs(M, N, K) if plain and M > 0 else 1
             part = _scratch(ws, (runs, M, N), torch.float32, x.device) if runs > 1 else None
             hipops.gemm_tiled(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
-                              y_rows=y_rows, glu=glu, shape=tile_shape, part=part)
-        else:
-            hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
-                             y_rows=y_rows, glu=glu)
+                              y_rows=y_rows, glu=glu, shape=tile_shape, part=part, act=act)
+            return
+        hipops.gemm_mfma(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
+                         y_rows=y_rows, glu=glu)
+        _act_after(y, M, y_rows, act)
         return
     if tiled:
         raise hipops.KernelError("linear: a weight in operand order met an input that the MFMA products do not take")
@@ -146,11 +152,23 @@ def linear(x, w, y, *, glu=False, offsets=None, n_groups=1, a_rows=None, a_scale
         if y.dtype == torch.float32:
             hipops.gemm_generic(x32, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                 a_scale=a_scale, y_rows=y_rows, glu=glu)
+            _act_after(y, M, y_rows, act)
         else:
             y32 = _scratch(ws, y.shape, torch.float32, y.device)
             hipops.gemm_generic(x32, w, y32, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows,
                                 a_scale=a_scale, y_rows=y_rows, glu=glu)
+            _act_after(y32, M, y_rows, act)
             hipops.convert(y32, y)
         return
     hipops.gemm_generic(x, w, y, M, N, K, offsets=offsets, n_groups=n_groups, a_rows=a_rows, a_scale=a_scale,
                         y_rows=y_rows, glu=glu)
+    _act_after(y, M, y_rows, act)
+
+
+def _act_after(y, M, y_rows, act):
+    """The activation as a pass of its own over the product's rows (the kernels that have no epilogue for it)."""
+    if act is None:
+        return
+    if y_rows is not None or not y.is_contiguous():
+        raise hipops.KernelError("linear: an activation after a product wants its rows in a row")
+    hipops.act_rows(y[:M], act)

@@ -34,8 +34,15 @@ class RMSNorm(Norm):
             and hipops.add_rmsnorm_can_project(self.width)
 
     def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, proj=None, proj_out=None,
-                normed=None):
-        """``normed``: a ``NormedIncrement``'s (y, weight, mult, eps), added like d1 and d2 after its own norm."""
+                normed=None, second=None):
+        """``normed``: a ``NormedIncrement``'s (y, weight, mult, eps), added like d1 and d2 after its own norm.
+        ``second`` = (another RMS norm of the same eps, its output): the same rows under that norm's
+        weights too, in one pass (a layer with two norms of one stream)."""
         hipops.add_rmsnorm(h, self.weight, self.eps, out=out, out32=out32, d1=d1, d2=d2, rows=rows,
                            n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h,
-                           proj=proj, proj_out=proj_out, normed=normed)
+                           proj=proj, proj_out=proj_out, normed=normed,
+                           w2=second[0].weight if second is not None else None, out2=second[1] if second is not None else None)
+
+    def pairs_with(self, other) -> bool:
+        """Whether ``other`` can be this norm's ``second``: the same kind, width and eps."""
+        return isinstance(other, RMSNorm) and other.width == self.width and other.eps == self.eps

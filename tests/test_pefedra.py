@@ -213,6 +213,30 @@ def test_activation_and_scaled_embedding(dtype, n):
     assert torch.equal(h.cpu(), table[ids.long()].float() * 12.5)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,M,N,K", [("float32", 9, 24, 40), ("bfloat16", 5, 64, 128), ("bfloat16", 100, 64, 128), ("bfloat16", 300, 1024, 256),
+                                         ("bfloat16", 200, 48, 72), ("bfloat16", 7, 20, 40), ("bfloat16", 40, 96, 64)])
+@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "silu"])
+def test_products_with_an_activation(dtype, M, N, K, act):
+    """act(x W^T) through every product kernel (in the epilogue where the kernel has one, else in a pass after it),
+    and a plain product right after it on the same thread."""
+    from spite_amd.parts.linear import linear, Weight
+    dt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(M + N)
+    x = (torch.randn(M, K, generator=g)).to(dt)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K) * 2).to(dt)
+    y = torch.empty(M, N, dtype=dt, device="cuda:0")
+    W = Weight(w.cuda())
+    linear(x.cuda(), W, y, act=act)
+    z = x.double() @ w.double().T
+    want = {"gelu": plain.gelu, "gelu_tanh": lambda v: 0.5 * v * (1 + torch.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v ** 3))),
+            "silu": lambda v: v * torch.sigmoid(v)}[act](z)
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert float((y.cpu().double() - want).abs().max()) <= tol * max(1.0, float(want.abs().max()))
+    linear(x.cuda(), W, y)
+    assert float((y.cpu().double() - z).abs().max()) <= tol * max(1.0, float(z.abs().max()))
+
+
 def _paged(rows, ps, perm, n_pages, heads, width, transposed):
     """rows[i]: [t, heads, width] of request i -> pages (NaN where nothing was written) and the block table."""
     n = len(rows)
