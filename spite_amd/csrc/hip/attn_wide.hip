@@ -16,7 +16,9 @@
 #define WIDE_NT 256
 
 // ------------------------------------------------------------------ projection row -> q, cache
-// One workgroup a token.  The row holds [HQ*D | GK*D | GV*Vd | ...] (`ld` elements to the next
+// A workgroup takes `hpb` heads of one token (query heads first, then key heads, then value heads; with
+// few tokens a step the heads are dealt to many workgroups, each of which forms the norm's sums over the
+// whole q or k part again).  The row holds [HQ*D | GK*D | GV*Vd | ...] (`ld` elements to the next
 // row).  x = row + bias; with `wq` / `wk` the q and the k region are each divided by the root mean
 // square of the whole region and multiplied by their weights; then the first `rot` elements
 // of every q and k head turn by pos * inv_freq[i] in pairs (i, i + rot/2); with `inv_freq_v` the
@@ -31,7 +33,7 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
                         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                         const int* __restrict__ positions, const int* __restrict__ slot_map,
                         const float* __restrict__ inv_freq, int rot, const float* __restrict__ inv_freq_v,
-                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp) {
+                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
     extern __shared__ float sm[];
     __shared__ float red[WIDE_NT / 64];
     const int rh = rot >> 1, vh = inv_freq_v ? (Vd >> 1) : 0;
@@ -45,26 +47,32 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
     const int Nq = HQ * D, Nk = GK * D;
     for (int i = tid; i < rh; i += WIDE_NT) sincosf(pos * inv_freq[i], &sn[i], &cs[i]);
     for (int i = tid; i < vh; i += WIDE_NT) sincosf(pos * inv_freq_v[i], &snv[i], &csv[i]);
+    const int slot = slot_map ? slot_map[t] : -1;
+    // this workgroup's heads [h_lo, h_hi) of the HQ + GK + GV; keys and values only where the token has a cache row
+    const int h_lo = blockIdx.y * hpb, h_end = h_lo + hpb;
+    const int qk_end = HQ + (slot >= 0 ? GK : 0);
+    const int qk_hi = h_end < qk_end ? h_end : qk_end;               // q and k heads [h_lo, qk_hi)
+    const int v_lo = (h_lo > HQ + GK ? h_lo : HQ + GK) - (HQ + GK);
+    const int v_hi = (h_end < HQ + GK + GV ? h_end : HQ + GK + GV) - (HQ + GK);       // value heads [v_lo, v_hi)
     float scale_q = 1.f, scale_k = 1.f;
-    if (wq) {
+    if (wq && h_lo < HQ) {
         float s = 0.f;
         for (int c = tid; c < Nq; c += WIDE_NT) { const float x = to_f32<T>(row[c]) + (bias ? bias[c] : 0.f); s += x * x; }
         scale_q = 1.0f / sqrtf(block_sum<WIDE_NT>(s, red) / (float)Nq + eps);
     }
-    if (wk) {
+    if (wk && h_lo < qk_end && h_end > HQ) {
         float s = 0.f;
         for (int c = tid; c < Nk; c += WIDE_NT) { const float x = to_f32<T>(row[Nq + c]) + (bias ? bias[Nq + c] : 0.f); s += x * x; }
         scale_k = 1.0f / sqrtf(block_sum<WIDE_NT>(s, red) / (float)Nk + eps);
     }
     __syncthreads();
-    const int slot = slot_map ? slot_map[t] : -1;
     const size_t page = slot >= 0 ? (size_t)(slot / ps) : 0;
     const int off = slot >= 0 ? slot % ps : 0;
     // a head of D elements is rh pairs and D - rot elements that pass through
     const int items = D - rh;
-    const int n_qk = (HQ + (slot >= 0 ? GK : 0)) * items;
+    const int n_qk = (qk_hi > h_lo ? qk_hi - h_lo : 0) * items;
     for (int it = tid; it < n_qk; it += WIDE_NT) {
-        const int hh = it / items, i = it % items;
+        const int hh = h_lo + it / items, i = it % items;
         const bool is_q = hh < HQ;
         const int base = hh * D;                       // the q and k regions follow each other in the row
         const float* wn = is_q ? wq : wk;
@@ -91,16 +99,16 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
             store(c, load(c));
         }
     }
-    for (int it = tid; it < (HQ + (slot >= 0 ? GK : 0)) * (Dp - D); it += WIDE_NT) {
-        const int hh = it / (Dp - D), c = D + it % (Dp - D);
+    for (int it = tid; it < (qk_hi > h_lo ? qk_hi - h_lo : 0) * (Dp - D); it += WIDE_NT) {
+        const int hh = h_lo + it / (Dp - D), c = D + it % (Dp - D);
         if (hh < HQ) q_out[((size_t)t * HQ + hh) * Dp + c] = from_f32<T>(0.f);
         else k_pages[(page * GK + (hh - HQ)) * (size_t)ps * Dp + sp_k_index(off, c, Dp, k_tiled)] = from_f32<T>(0.f);
     }
     if (slot < 0) return;
     const int vitems = Vd - vh;
     const int vbase = Nq + Nk;
-    for (int it = tid; it < GV * vitems; it += WIDE_NT) {
-        const int g = it / vitems, i = it % vitems;
+    for (int it = tid; it < (v_hi > v_lo ? v_hi - v_lo : 0) * vitems; it += WIDE_NT) {
+        const int g = v_lo + it / vitems, i = it % vitems;
         T* slab = v_pages + (page * GV + g) * (size_t)Vd * ps;
         auto load = [&](int c) { return to_f32<T>(row[vbase + g * Vd + c]) + (bias ? bias[vbase + g * Vd + c] : 0.f); };
         if (i < vh) {
@@ -133,12 +141,19 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
     if (T == 0) return 0;
     const size_t sh = (size_t)(rot + (inv_freq_v ? Vd : 0)) * sizeof(float);
     SP_REQUIRE(sh <= 48 * 1024, "qkv_prepare: heads too wide");
+    // heads a workgroup: all of a token's for many tokens; for few, so many that about two workgroups a compute unit run
+    const int heads = HQ + GK + GV;
+    long hpb = ((long)heads * T + 2 * sp_cu_count() - 1) / (2 * sp_cu_count());
+    if (hpb < 1) hpb = 1;
+    if (hpb > 16) hpb = 16;                          // (more waves in flight hide the rows' 2-byte loads and stores)
+    if (hpb > heads) hpb = heads;
+    const dim3 grid(T, (unsigned)((heads + hpb - 1) / hpb));
     if (dtype == SP_F32)
-        qkv_prepare_kernel<float><<<T, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
-            (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp);
+        qkv_prepare_kernel<float><<<grid, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
+            (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
     else if (dtype == SP_BF16)
-        qkv_prepare_kernel<bf16><<<T, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp);
+        qkv_prepare_kernel<bf16><<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
     else return sp_fail("qkv_prepare: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("qkv_prepare");
     return 0;

@@ -157,7 +157,7 @@ void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restr
         }
         if (a_scale) { const float sc = a_scale[s]; v *= sc; u *= sc; }
         if (GLU) v = sp_gate_act(v, act, true) * u;
-        else if (act < 0) v = sp_unary(v, -act);                 // a plain product with an activation of its own
+        else if (act < 0) v = sp_unary(v, -act, true);                 // a plain product with an activation of its own
         const size_t yr = y_rows ? (size_t)y_rows[s] : (size_t)s;
         Y[yr * ldy + n] = from_f32<TY>(v);
     }

@@ -279,7 +279,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ X, int ldx, const bf16* __restri
                 for (int i = 0; i < 4; ++i) v[i] = acc[a][b][i] * sc;
                 if (act < 0) {                                   // a plain product with an activation of its own
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] = sp_unary(v[i], -act);
+                    for (int i = 0; i < 4; ++i) v[i] = sp_unary(v[i], -act, true);
                 }
                 put4(yrow, ncol[a] + q * 4, v);
             }

@@ -17,17 +17,34 @@ void token_shift_kernel(const float* __restrict__ x, TO* __restrict__ y, const f
     const int first = cu_seqlens[e], last = cu_seqlens[e + 1] - 1;
     const float* xr = x + (size_t)t * d;
     TO* yr = y + (size_t)t * d;
-    if (t != first) {
-        const float* xp = xr - d;
-        for (int c = threadIdx.x; c < d; c += 256) { const float a = xr[c]; yr[c] = from_f32<TO>(a + (xp[c] - a) * w[c]); }
+    const int c0 = blockIdx.y * 1024;                      // a workgroup takes 1,024 elements of the row
+    const int c1 = c0 + 1024 < d ? c0 + 1024 : d;
+    float* sr = t == first ? state + (size_t)seq_slots[e] * d : nullptr;
+    const float* xp = t == first ? sr : xr - d;
+    const float* xl = x + (size_t)last * d;
+    if ((d & 3) == 0) {                                    // (rows of fp32 start on 16 bytes then)
+        const int c = c0 + threadIdx.x * 4;
+        if (c >= c1) return;
+        const f32x4 a = *(const f32x4*)(xr + c), b = *(const f32x4*)(xp + c), ww = *(const f32x4*)(w + c);
+        const f32x4 keep4 = (sr && keep) ? *(const f32x4*)(xl + c) : a;
+        f32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = a[i] + (b[i] - a[i]) * ww[i];
+        if constexpr (sizeof(TO) == 2) {
+            bf16x4 o4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = (bf16)o[i];
+            *(bf16x4*)((bf16*)yr + c) = o4;
+        } else {
+            *(f32x4*)((float*)yr + c) = o;
+        }
+        if (sr && keep) *(f32x4*)(sr + c) = keep4;
         return;
     }
-    float* sr = state + (size_t)seq_slots[e] * d;
-    const float* xl = x + (size_t)last * d;
-    for (int c = threadIdx.x; c < d; c += 256) {
+    for (int c = c0 + threadIdx.x; c < c1; c += 256) {
         const float a = xr[c];
-        yr[c] = from_f32<TO>(a + (sr[c] - a) * w[c]);
-        if (keep) sr[c] = xl[c];
+        yr[c] = from_f32<TO>(a + (xp[c] - a) * w[c]);
+        if (sr && keep) sr[c] = xl[c];
     }
 }
 
@@ -35,9 +52,13 @@ extern "C" int spite_token_shift(const float* x, void* y, int y_dtype, const flo
                                  const int* seq_of_token, const int* cu_seqlens, const int* seq_slots, int T, int d,
                                  int keep, hipStream_t st) {
     SP_REQUIRE(T >= 0 && d > 0, "token_shift: bad sizes T=%d d=%d", T, d);
+    SP_REQUIRE((d + 1023) / 1024 <= 65535, "token_shift: rows of %d", d);
     if (T == 0) return 0;
-    if (y_dtype == SP_F32) token_shift_kernel<float><<<T, 256, 0, st>>>(x, (float*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
-    else if (y_dtype == SP_BF16) token_shift_kernel<bf16><<<T, 256, 0, st>>>(x, (bf16*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
+    const dim3 grid(T, (d + 1023) / 1024);
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    SP_REQUIRE((d & 3) != 0 || (al(x) && al(y) && al(w) && al(state)), "token_shift: rows must start on 16 bytes");
+    if (y_dtype == SP_F32) token_shift_kernel<float><<<grid, 256, 0, st>>>(x, (float*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
+    else if (y_dtype == SP_BF16) token_shift_kernel<bf16><<<grid, 256, 0, st>>>(x, (bf16*)y, w, state, seq_of_token, cu_seqlens, seq_slots, d, keep);
     else return sp_fail("token_shift: unknown dtype %d", y_dtype);
     SP_LAUNCH_CHECK("token_shift");
     return 0;
@@ -49,7 +70,7 @@ template <typename T>
 __global__ __launch_bounds__(256)
 void act_rows_kernel(T* __restrict__ x, size_t n, int act) {
     const size_t stride = (size_t)gridDim.x * 256;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) x[i] = from_f32<T>(sp_unary(to_f32<T>(x[i]), act));
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) x[i] = from_f32<T>(sp_unary(to_f32<T>(x[i]), act, false));
 }
 
 // eight bfloat16 a thread and step
@@ -59,7 +80,7 @@ void act_rows_bf16x8_kernel(bf16x8* __restrict__ x, size_t n8, int act) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
         bf16x8 v = x[i];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = (bf16)sp_unary((float)v[e], act);
+        for (int e = 0; e < 8; ++e) v[e] = (bf16)sp_unary((float)v[e], act, false);
         x[i] = v;
     }
 }
