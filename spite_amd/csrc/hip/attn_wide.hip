@@ -122,6 +122,104 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
     }
 }
 
+// The same for bfloat16 rows whose sizes let a thread move four elements at a time (D, Dp, the row stride
+// and the distance between a pair's elements multiples of four): 8-byte loads and stores for queries and
+// keys (four elements in a row stay in a row in operand order too), the values one by one as above.  Every
+// value is computed by the same operations as in the kernel above.
+__global__ __launch_bounds__(WIDE_NT)
+void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* __restrict__ bias,
+                            const float* __restrict__ wq, const float* __restrict__ wk, float eps,
+                            bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                            const int* __restrict__ positions, const int* __restrict__ slot_map,
+                            const float* __restrict__ inv_freq, int rot, const float* __restrict__ inv_freq_v,
+                            int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    __shared__ float red[WIDE_NT / 64];
+    const int rh = rot >> 1, vh = inv_freq_v ? (Vd >> 1) : 0;
+    float* cs = sm;
+    float* sn = cs + rh;
+    float* csv = sn + rh;
+    float* snv = csv + vh;
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float pos = (float)positions[t];
+    const bf16* row = qkv + (size_t)t * ld;
+    const int Nq = HQ * D, Nk = GK * D;
+    for (int i = tid; i < rh; i += WIDE_NT) sincosf(pos * inv_freq[i], &sn[i], &cs[i]);
+    for (int i = tid; i < vh; i += WIDE_NT) sincosf(pos * inv_freq_v[i], &snv[i], &csv[i]);
+    const int slot = slot_map ? slot_map[t] : -1;
+    const int h_lo = blockIdx.y * hpb, h_end = h_lo + hpb;
+    const int qk_end = HQ + (slot >= 0 ? GK : 0);
+    const int qk_hi = h_end < qk_end ? h_end : qk_end;
+    const int v_lo = (h_lo > HQ + GK ? h_lo : HQ + GK) - (HQ + GK);
+    const int v_hi = (h_end < HQ + GK + GV ? h_end : HQ + GK + GV) - (HQ + GK);
+    auto row4 = [&](int c) {                               // four elements of the row from c on, with their bias
+        const bf16x4 r = *(const bf16x4*)(row + c);
+        f32x4 x = {(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+        if (bias) x += *(const f32x4*)(bias + c);
+        return x;
+    };
+    auto sumsq = [&](int from, int n) {
+        float s = 0.f;
+        for (int c = tid * 4; c < n; c += WIDE_NT * 4) { const f32x4 x = row4(from + c); s += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3]; }
+        return block_sum<WIDE_NT>(s, red);
+    };
+    float scale_q = 1.f, scale_k = 1.f;
+    if (wq && h_lo < HQ) scale_q = 1.0f / sqrtf(sumsq(0, Nq) / (float)Nq + eps);
+    if (wk && h_lo < qk_end && h_end > HQ) scale_k = 1.0f / sqrtf(sumsq(Nq, Nk) / (float)Nk + eps);
+    __syncthreads();
+    const size_t page = slot >= 0 ? (size_t)(slot / ps) : 0;
+    const int off = slot >= 0 ? slot % ps : 0;
+    // a head in groups of four: pairs that turn, elements that pass through, zeros behind D
+    const int pq = rh >> 2, sq = (D - rot) >> 2, zq = (Dp - D) >> 2, QI = pq + sq + zq;
+    const int n_qk = (qk_hi > h_lo ? qk_hi - h_lo : 0) * QI;
+    for (int it = tid; it < n_qk; it += WIDE_NT) {
+        const int hh = h_lo + it / QI, j = it % QI;
+        const bool is_q = hh < HQ;
+        const int base = hh * D;
+        const float* wn = is_q ? wq : wk;
+        const float sc = is_q ? scale_q : scale_k;
+        const int wbase = is_q ? base : base - Nq;
+        auto load = [&](int c) {
+            f32x4 x = row4(base + c);
+            if (wn) { const f32x4 ww = *(const f32x4*)(wn + wbase + c); x = x * sc * ww; }
+            return x;
+        };
+        bf16* dst = is_q ? q_out + ((size_t)t * HQ + hh) * Dp : k_pages + (page * GK + (hh - HQ)) * (size_t)ps * Dp;
+        auto store = [&](int c, const f32x4& v) {
+            const bf16x4 o = {(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+            *(bf16x4*)(dst + (is_q ? (size_t)c : sp_k_index(off, c, Dp, k_tiled))) = o;
+        };
+        if (j < pq) {
+            const int i = j * 4;
+            const f32x4 a = load(i), b = load(i + rh);
+            const f32x4 c4 = *(const f32x4*)(cs + i), s4 = *(const f32x4*)(sn + i);
+            store(i, a * c4 - b * s4);
+            store(i + rh, b * c4 + a * s4);
+        } else if (j < pq + sq) {
+            const int c = rot + (j - pq) * 4;
+            store(c, load(c));
+        } else {
+            store(D + (j - pq - sq) * 4, f32x4{0.f, 0.f, 0.f, 0.f});
+        }
+    }
+    if (slot < 0) return;
+    const int vitems = Vd - vh;
+    const int vbase = Nq + Nk;
+    for (int it = tid; it < (v_hi > v_lo ? v_hi - v_lo : 0) * vitems; it += WIDE_NT) {
+        const int g = v_lo + it / vitems, i = it % vitems;
+        bf16* slab = v_pages + (page * GV + g) * (size_t)Vd * ps;
+        auto load = [&](int c) { return (float)row[vbase + g * Vd + c] + (bias ? bias[vbase + g * Vd + c] : 0.f); };
+        if (i < vh) {
+            const float a = load(i), b = load(i + vh);
+            slab[sp_v_index(i, off, Vd, ps, v_tiled)] = (bf16)(a * csv[i] - b * snv[i]);
+            slab[sp_v_index(i + vh, off, Vd, ps, v_tiled)] = (bf16)(b * csv[i] + a * snv[i]);
+        } else {
+            const int c = 2 * vh + (i - vh);
+            slab[sp_v_index(c, off, Vd, ps, v_tiled)] = (bf16)load(c);
+        }
+    }
+}
+
 extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float* bias, const float* wq, const float* wk,
                                  float eps, void* q_out, void* k_pages, void* v_pages, const int* positions,
                                  const int* slot_map, const float* inv_freq, int rot, const float* inv_freq_v,
@@ -148,6 +246,15 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
     if (hpb > 16) hpb = 16;                          // (more waves in flight hide the rows' 2-byte loads and stores)
     if (hpb > heads) hpb = heads;
     const dim3 grid(T, (unsigned)((heads + hpb - 1) / hpb));
+    auto al = [](const void* p, int a) { return ((uintptr_t)p & (a - 1)) == 0; };
+    if (dtype == SP_BF16 && D % 4 == 0 && Dp % 4 == 0 && rot % 8 == 0 && ld % 4 == 0 && al(qkv, 8) && al(q_out, 8) && al(k_pages, 8)
+        && al(bias, 16) && al(wq, 16) && al(wk, 16)) {
+        // (the sine and cosine tables are read four at a time: the second starts rot/2 floats behind the first)
+        qkv_prepare_vec_kernel<<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+        SP_LAUNCH_CHECK("qkv_prepare");
+        return 0;
+    }
     if (dtype == SP_F32)
         qkv_prepare_kernel<float><<<grid, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
             (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
