@@ -594,6 +594,51 @@ def test_far_keys_and_long_decoding(tmp_path, kind):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,wide", [("float32", False), ("bfloat16", True)])
+def test_one_far_key_stands_out(tmp_path, dtype, wide):
+    """One token, seen once at position 3, whose key every later query of the first score map scores far above all
+    others (a query bias on an element that does not turn, and a key row along that token's normed embedding):
+    hundreds of keys later, in the prompt and in decoded tokens, the result is that key's value.  Without it the
+    logits are others altogether, which the test shows first."""
+    cfg = _one_layer("attention", None, wide=wide)
+    cfg["layers"][0]["mixer"]["scale"] = 0.25
+    mx = cfg["layers"][0]["mixer"]
+    Hh, G, D, d, special, gain = mx["heads"], mx["kv_heads"], mx["dim"], cfg["width"], 7, 5.0
+    t = planted(cfg, 3, gain=1.0)
+    t["l0.shift"] = torch.zeros(d)
+    h = t["embed"][special].double() * cfg["embedding"]["scale"]
+    h = plain.norm(h, t["l0.norm1"].double(), cfg["norm"]["eps"])
+    u = (h / h.norm()).float()
+    c0 = D - 1                                                     # behind the elements that turn
+    for hh in range(Hh):
+        t["l0.mix.q"][(hh * 2) * D + c0] = 0.0
+        t["l0.mix.q.b"][(hh * 2) * D + c0] = gain
+    for g in range(G):
+        t["l0.mix.k"][(g * 2) * D + c0] = gain * u
+        t["l0.mix.k.b"][(g * 2) * D + c0] = 0.0
+    from spite_amd.weights.random_init import write_random_model
+    write_random_model(str(tmp_path), cfg, 3, dtype=dtype, overrides=t)
+    weights = H.read_weights(str(tmp_path))
+    toks = [x if x != special else special + 1 for x in H.random_tokens(64, 330, 9)]
+    toks[3] = special
+    without = list(toks)
+    without[3] = special + 1
+    ref, other = plain.forward(cfg, weights, toks), plain.forward(cfg, weights, without)
+    scale = float(ref.abs().max())
+    assert float((ref[300:] - other[300:]).abs().max()) > 0.2 * scale          # the far key decides
+    from spite_amd import Engine
+    eng = Engine(str(tmp_path), dtype=dtype, page_size=32 if wide else 8, cache_tokens=512, max_requests=2, device="cuda:0")
+    if wide:
+        assert not eng.slow_paths, eng.slow_paths
+    poison(eng)
+    steps = H.schedule_tail_one_by_one({"a": toks}, tail=40)
+    got = H.collect(steps, H.run_trace_inprocess(eng, steps), 64)
+    rows = {("a", i): ref[i].float().numpy() for i in range(len(toks))}
+    err, where = H.max_diff(got, rows)
+    assert err <= (2e-4 if dtype == "float32" else 0.05) * scale, f"{err} at {where} (scale {scale})"
+
+
+@pytest.mark.gpu
 def test_a_slot_used_again_starts_from_zeros(models):
     """A request that takes the slot (and the pages) of a finished one reads nothing of it: its first
     token's shift sees zeros, whatever the slot's state row held."""
