@@ -232,11 +232,11 @@ DESIGN_SIZES = {
 def pefedra_configs(sz, layers, window, vocab):
     H = sz["heads"]
     gated = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
-             "rot": {"base": 500000.0, "dims": 64}}
-    two_maps = {"heads": H // 2, "kv_heads": max(1, H // 8), "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.5,
-                "mask": {"size": window}, "rot": {"base": 50000.0, "dims": 64, "scaling": {"factor": 8.0}}}
+             "rot": {"base": 1000000.0, "dims": 64}}
+    two_maps = {"heads": H // 2, "kv_heads": max(1, H // 8), "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.3,
+                "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0}}}
     mlp = {"kind": "dense", "ff": sz["dense_ff"] * 3 // 2}
-    pefedra = {"architecture": "Pefedra", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
+    pefedra = {"architecture": "Pefedra", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
                "torch_dtype": "bfloat16",
                "layers": [{"type": "attention", "mixer": two_maps, "mlp": mlp} if i % 4 == 2 else
                           {"type": "attention_2", "mixer": gated, "mlp": mlp} for i in range(layers)]}
